@@ -1,0 +1,105 @@
+/*
+ * spingalett_hip.h — C ABI of the kernel translation unit (hip_forward.hip).
+ *
+ * This is the boundary the reference's own glue would bind: plain pointers
+ * and sizes, int status (0 = ok), no exceptions, no HIP types.  Each entry
+ * cites the reference code whose work it takes over.
+ *
+ * Data held on the device per net: for every layer the weight array and the
+ * bias array exactly as serialized in a .nn file (Serialize.c:87-193): raw
+ * FP32, u16 FP16/BF16 codes, or packed INT8/INT4/INT2 codes; the f32 scale
+ * that precedes the integer formats travels as `max_val`.  Kernels unpack in
+ * their inner loops; no FP32 expansion of the weights exists on the device.
+ */
+#ifndef SPINGALETT_HIP_ABI_H
+#define SPINGALETT_HIP_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPHIP_API __attribute__((visibility("default")))
+
+typedef struct sphip_net sphip_net;
+
+/* Shape of a net: what new_spingalett()/layer() accumulate in NeuralNetwork
+ * (Spingalett.h:109-136) reduced to what inference needs.
+ *   precision : PrecisionMode value of every array (Spingalett.h:93-101)
+ *   act[l]    : ActivationFunction of layer l+1 (Spingalett.h:38-47)       */
+typedef struct {
+    uint32_t        layers;      /* including the input layer, >= 2 */
+    const uint32_t *topology;    /* [layers]                        */
+    const uint8_t  *act;         /* [layers-1]                      */
+    uint8_t         precision;
+} sphip_desc;
+
+/* flags of sphip_forward */
+#define SPHIP_X_ON_DEVICE   1u   /* x is a device pointer                       */
+#define SPHIP_Y_ON_DEVICE   2u   /* y is a device pointer (call does not wait)  */
+#define SPHIP_KEEP_LAYERS   4u   /* keep every layer's activations (n must be 1)*/
+#define SPHIP_FORCE_GEMM    8u   /* use the matrix-core path whatever n is      */
+#define SPHIP_FORCE_GEMV   16u   /* use the vector path (n <= 64)               */
+
+SPHIP_API int  sphip_device_count(void);
+SPHIP_API const char *sphip_last_error_string(void);   /* per thread */
+
+/* Replaces the per-net allocation done by layer_struct_arguments
+ * (Network.c:83-105) on the device side. */
+SPHIP_API int  sphip_create(const sphip_desc *desc, sphip_net **out);
+SPHIP_API void sphip_destroy(sphip_net *net);           /* free_network, Network.c:283 */
+
+/* Replaces read_array_compressed (Serialize.c:195-297): instead of expanding
+ * to FP32 the serialized codes are copied to the device as they are.
+ *   which   : 0 weights of layer l (topology[l]*topology[l+1] elements), 1 biases
+ *   codes   : the array's bytes after the 4-byte scale (host memory)
+ *   max_val : the scale read from the file (ignored for FP32/FP16/BF16)     */
+SPHIP_API int  sphip_upload_array(sphip_net *net, uint32_t l, int which,
+                                  const void *codes, size_t bytes, float max_val);
+
+/* Replaces forward_struct_arguments (Network.c:202-251) for n = 1 and
+ * batch_forward (Training.c:313-345) for n > 1:
+ *   per layer  y = act(b + W x), x row-major [n][topology[0]], y row-major
+ *   [n][topology[last]], FP32.  n <= 64 runs the vector (GEMV) kernels in
+ *   FP32 arithmetic; larger n runs the matrix-core kernels with 16-bit
+ *   activations (FP32 weights always use FP32 arithmetic). */
+SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y,
+                             uint32_t flags);
+/* After a SPHIP_KEEP_LAYERS forward: copies all layers' activations to a host
+ * array laid out like NeuralNetwork.neurons (Network.c:16-32). */
+SPHIP_API int  sphip_read_layers(sphip_net *net, float *host_neurons);
+
+/* The device form of the decoders in read_array_compressed
+ * (Serialize.c:195-297) and fp16_to_float / bf16_to_float (:45-85): writes the
+ * FP32 value of every element of one array to host memory.
+ *   mode 0: ((float)q/d)*max evaluated as written; 1: q*(max*(1/d)).       */
+SPHIP_API int  sphip_decode(sphip_net *net, uint32_t l, int which, int mode,
+                            float *host_out);
+
+SPHIP_API int  sphip_synchronize(void);
+
+/* ---- measurement helpers (benchmark harness; not part of the data path) ---- */
+SPHIP_API int  sphip_malloc(void **dptr, size_t bytes);
+SPHIP_API int  sphip_free(void *dptr);
+SPHIP_API int  sphip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+SPHIP_API int  sphip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+/* A second device copy of a net's arrays (so a timing loop can rotate over
+ * copies larger than the last-level cache). */
+SPHIP_API int  sphip_clone(const sphip_net *src, sphip_net **out);
+/* Runs `iters` forwards of n samples, rotating over nets[0..count), between two
+ * HIP events recorded on the library's stream; *ms = total elapsed. */
+SPHIP_API int  sphip_time_forward(sphip_net *const *nets, int count, const float *d_x,
+                                  uint32_t n, float *d_y, uint32_t flags, int iters, float *ms);
+/* Same for the main kernel of one layer only (layer index 1..layers-1). */
+SPHIP_API int  sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer,
+                                uint32_t n, uint32_t flags, int iters, float *ms);
+/* Name of the kernel sphip_time_layer launches for that layer and n. */
+SPHIP_API const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n,
+                                              uint32_t flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPINGALETT_HIP_ABI_H */

@@ -1,0 +1,113 @@
+/*
+ * sp_oracle.h — CPU restatement of Spingalett's quantized-load + forward path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library links, loads or
+ * calls this code; it exists so that tests, the smoke check and the benchmark's
+ * CPU-baseline leg have an independent statement of what the reference
+ * computes.  Every function cites the reference lines it restates
+ * (paths relative to the reference tree).
+ *
+ * Pin status (what fixes each function besides this restatement itself):
+ *   orc_fp16_to_f32 / orc_bf16_to_f32 ....... pinned: all 65,536 codes against
+ *        numpy's IEEE half->single conversion plus the NaN-canonicalisation
+ *        rule, and against the closed form code<<16.
+ *   orc_decode_array ........................ pinned: every INT8/INT4/INT2 code
+ *        against IEEE float32 arithmetic done by numpy, hand-derived
+ *        known-answer bytes (nibble/crumb order, sign extension, max<=0 -> 0).
+ *   orc_encode_array ........................ pinned: round trips, hand-derived
+ *        known answers (ties round half away from zero, INT4 clamp, ternary
+ *        thresholds, FP16/BF16 truncation).
+ *   orc_parse / orc_serialize ............... pinned: hand-assembled files and
+ *        byte counts (8+5L header, 16+5L with optimizer block).
+ *   orc_forward_* ........................... pinned: float64 brute force on
+ *        small nets, numpy matmul + scipy special functions at size, closed
+ *        forms for the piecewise-linear activations, softmax invariants.
+ *   The last-bit summation order of the reference's BLAS / AVX dot product is
+ *   deliberately not reproduced (tolerance 1e-4, not bits).
+ */
+#ifndef SP_ORACLE_H
+#define SP_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* enum values follow Include/Spingalett/Spingalett.h:38-47 and :93-101 */
+enum { ORC_ACT_SIGMOID = 0, ORC_ACT_RELU, ORC_ACT_TANH, ORC_ACT_LEAKY_RELU,
+       ORC_ACT_FOO52, ORC_ACT_SOFTMAX, ORC_ACT_NONE, ORC_ACT_COUNT };
+enum { ORC_PREC_F32 = 0, ORC_PREC_F16, ORC_PREC_BF16, ORC_PREC_I8,
+       ORC_PREC_I4, ORC_PREC_I2, ORC_PREC_COUNT };
+
+/* How the INT8 / INT4 decode expression is evaluated.
+ *   STRICT : ((float)q / d) * max  exactly as written (Serialize.c:233,258).
+ *   RELEASE: (float)q * (max * (1.0f/d)) — what the reference's own Release
+ *            flag set (-freciprocal-math -fassociative-math,
+ *            CMakeLists.txt:143-157) turns that expression into. */
+enum { ORC_DEQUANT_STRICT = 0, ORC_DEQUANT_RELEASE = 1 };
+
+typedef struct {
+    uint32_t  layers;          /* including the input layer            */
+    uint32_t *topology;        /* [layers]                             */
+    uint8_t  *act;             /* [layers-1]                           */
+    uint8_t   loss;
+    uint8_t   has_optimizer;
+    uint8_t   precision;       /* of the file the net was parsed from  */
+    uint64_t  time_step;
+    uint64_t *woff;            /* [layers-1] offsets into weights      */
+    uint64_t *boff;            /* [layers-1] offsets into biases       */
+    uint64_t  total_weights, total_biases;
+    float    *weights;         /* row-major [out][in] per layer        */
+    float    *biases;
+    int       truncated;       /* payload ended early (Serialize.c:596) */
+} orc_net;
+
+/* --- scalar codecs (Serialize.c:12-85) --- */
+float    orc_fp16_to_f32(uint16_t h);
+uint16_t orc_f32_to_fp16(float x);
+float    orc_bf16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float x);
+
+/* --- array codecs (Serialize.c:87-297) --- */
+size_t orc_array_bytes(uint32_t n, int precision);
+/* returns bytes consumed, 0 when `avail` is too small */
+size_t orc_decode_array(const uint8_t *src, size_t avail, uint32_t n,
+                        int precision, int mode, float *dst);
+/* returns bytes written (dst must hold orc_array_bytes) */
+size_t orc_encode_array(const float *src, uint32_t n, int precision, uint8_t *dst);
+
+/* --- file (Serialize.c:307-609) --- */
+orc_net *orc_new(uint32_t layers, const uint32_t *topology, const uint8_t *act);
+void     orc_free(orc_net *net);
+/* err: 0 ok, 1 short header, 2 bad version, 3 layers<2, 4 bad loss,
+ *      5 bad precision, 6 bad activation */
+orc_net *orc_parse(const uint8_t *buf, size_t len, int mode, int *err);
+size_t   orc_serialized_size(const orc_net *net, int precision, int with_optimizer);
+size_t   orc_serialize(const orc_net *net, int precision, int with_optimizer,
+                       uint8_t *dst);
+
+/* --- activations (Activation.c:5-38, SIMD.c:21-88) --- */
+float orc_activate(float x, int act);
+void  orc_softmax(float *row, uint32_t n);
+void  orc_apply_activation(float *data, uint64_t rows, uint32_t width, int act);
+
+/* --- forward --- */
+/* Network.c:202-251, scalar: y = act(b + W x); out holds the last layer. */
+void orc_forward_single(const orc_net *net, const float *x, float *out);
+/* Training.c:313-345: C = A W^T, C += 1 (x) b, activation; FP32, k-sequential. */
+void orc_forward_batch(const orc_net *net, const float *X, uint32_t N, float *out);
+/* Same mathematics in float64 end to end (brute-force check, not the reference). */
+void orc_forward_batch_f64(const orc_net *net, const float *X, uint32_t N, double *out);
+
+/* CPU-baseline leg: same call sequence with a threaded sgemm.  sgemm_fn is a
+ * cblas_sgemm-compatible pointer found at run time, or NULL for the built-in
+ * OpenMP kernel.  Returns seconds per call averaged over `iters`. */
+double orc_time_forward_batch(const orc_net *net, const float *X, uint32_t N,
+                              float *out, int iters, void *sgemm_fn, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,1199 @@
+// hip_forward.hip — gfx950 kernels and the C ABI of spingalett_hip.h.
+//
+// One translation unit holds every HIP runtime call and every kernel of the
+// inference path:
+//   sp_decode_*      element decoders (bit-exact with Serialize.c:45-85,195-297)
+//   sp_gemv_*        n <= 64: FP32-arithmetic dequant GEMV, fused bias+activation
+//   sp_gemm16_*      n  > 64: LDS-tiled dequant-to-16-bit MFMA GEMM, fused epilogue
+//   sp_gemm32_f32    n  > 64 with FP32 weights: FP32 MFMA GEMM
+//   sp_softmax_rows  per-sample softmax (Activation.c:5-21)
+// Weights stay in their serialized form on the device; row-major [out][in]
+// (Private.h:16), element i of an INT4 array in nibble i&1 of byte i/2, element
+// i of an INT2 array at bits 2(i%4) of byte i/4 (Serialize.c:148-152,181-183).
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "spingalett_hip.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// formats and small helpers
+// ---------------------------------------------------------------------------
+enum : int { F32 = 0, F16 = 1, BF16 = 2, I8 = 3, I4 = 4, I2 = 5, NFMT = 6 };
+enum : int { A_SIGMOID = 0, A_RELU, A_TANH, A_LEAKY, A_FOO52, A_SOFTMAX, A_NONE, A_COUNT };
+
+constexpr int kWave = 64;
+
+__host__ __device__ constexpr int fmt_bits(int f)
+{
+    return f == F32 ? 32 : (f == F16 || f == BF16) ? 16 : f == I8 ? 8 : f == I4 ? 4 : 2;
+}
+
+size_t fmt_bytes(int f, uint64_t n)
+{
+    return (size_t)((n * (uint64_t)fmt_bits(f) + 7u) / 8u);
+}
+
+// divisor d of the integer formats: w = (q / d) * max   (Serialize.c:233,258,285)
+float fmt_divisor(int f) { return f == I8 ? 127.0f : f == I4 ? 7.0f : 1.0f; }
+
+// folded scale used by the arithmetic kernels: w = q * scale
+float fmt_scale(int f, float max_val)
+{
+    if (f == F32 || f == F16 || f == BF16) return 1.0f;
+    if (!(max_val > 0.0f)) return 0.0f;            // Serialize.c:231-236: zeros
+    return (float)((double)max_val / (double)fmt_divisor(f));
+}
+
+thread_local char g_err[512] = "";
+
+int fail_msg(const char *msg)
+{
+    snprintf(g_err, sizeof g_err, "%s", msg);
+    return 1;
+}
+
+int fail_hip(const char *what, hipError_t e)
+{
+    snprintf(g_err, sizeof g_err, "%s: %s", what, hipGetErrorString(e));
+    return 1;
+}
+
+#define HCHECK(expr)                                              \
+    do {                                                          \
+        hipError_t e_ = (expr);                                   \
+        if (e_ != hipSuccess) return fail_hip(#expr, e_);         \
+    } while (0)
+
+hipStream_t g_stream = nullptr;
+
+int ensure_stream()
+{
+    if (g_stream) return 0;
+    int cnt = 0;
+    HCHECK(hipGetDeviceCount(&cnt));
+    if (cnt <= 0) return fail_msg("no HIP device");
+    HCHECK(hipSetDevice(0));
+    HCHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// device-side element access
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float bits_to_float(uint32_t u) { return __uint_as_float(u); }
+
+// binary16 -> binary32, integer arithmetic only; any NaN becomes the quiet NaN
+// of the same sign (Serialize.c:45-72).
+__device__ __forceinline__ float half_bits_to_float_exact(uint32_t h)
+{
+    uint32_t s = (h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 31u;
+    uint32_t m = h & 1023u;
+    uint32_t f;
+    if (e == 31u) {
+        f = s | (m ? 0x7FC00000u : 0x7F800000u);
+    } else if (e != 0u) {
+        f = s | ((e + 112u) << 23) | (m << 13);
+    } else if (m == 0u) {
+        f = s;
+    } else {
+        int lz = __clz((int)m) - 21;               // shifts until bit 10 is set
+        m = (m << lz) & 1023u;
+        f = s | ((uint32_t)(113 - lz) << 23) | (m << 13);
+    }
+    return bits_to_float(f);
+}
+
+// integer code of element i of a packed INT array
+template <int FMT>
+__device__ __forceinline__ int int_code(const uint8_t *codes, uint64_t i)
+{
+    if constexpr (FMT == I8) {
+        return (int)(int8_t)codes[i];
+    } else if constexpr (FMT == I4) {
+        uint32_t byte = codes[i >> 1];
+        uint32_t nib = (i & 1u) ? (byte >> 4) : (byte & 15u);
+        return (int)nib - (int)((nib & 8u) << 1);
+    } else {
+        uint32_t c = (codes[i >> 2] >> ((i & 3u) * 2u)) & 3u;
+        return (int)c - (int)((c & 2u) << 1);
+    }
+}
+
+// unscaled value of element i: the float itself for FP formats, (float)q for INT
+template <int FMT>
+__device__ __forceinline__ float elem_value(const uint8_t *codes, uint64_t i)
+{
+    if constexpr (FMT == F32) {
+        return reinterpret_cast<const float *>(codes)[i];
+    } else if constexpr (FMT == F16) {
+        return half_bits_to_float_exact(reinterpret_cast<const uint16_t *>(codes)[i]);
+    } else if constexpr (FMT == BF16) {
+        return bits_to_float((uint32_t)reinterpret_cast<const uint16_t *>(codes)[i] << 16);
+    } else {
+        return (float)int_code<FMT>(codes, i);
+    }
+}
+
+__device__ __forceinline__ float elem_value_rt(int fmt, const uint8_t *codes, uint64_t i)
+{
+    switch (fmt) {
+    case F32:  return elem_value<F32>(codes, i);
+    case F16:  return elem_value<F16>(codes, i);
+    case BF16: return elem_value<BF16>(codes, i);
+    case I8:   return elem_value<I8>(codes, i);
+    case I4:   return elem_value<I4>(codes, i);
+    default:   return elem_value<I2>(codes, i);
+    }
+}
+
+// Activation.c:23-38 (leak factor fixed at 0.01f).  Softmax is a row operation
+// and handled by sp_softmax_rows.
+__device__ __forceinline__ float apply_act(float x, int act)
+{
+    switch (act) {
+    case A_SIGMOID: return 1.0f / (1.0f + expf(-x));
+    case A_RELU:    return x > 0.0f ? x : 0.0f;
+    case A_TANH:    return tanhf(x);
+    case A_LEAKY:   return x > 0.0f ? x : 0.01f * x;
+    case A_FOO52:   return x > 1.0f ? 1.0f + 0.01f * (x - 1.0f) : (x < 0.0f ? 0.01f * x : x);
+    default:        return x;
+    }
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
+{
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_sat(float x)
+{
+    if (x != x) return (uint16_t)0x7E00u;
+    x = fminf(fmaxf(x, -65504.0f), 65504.0f);
+    _Float16 h = (_Float16)x;
+    uint16_t r;
+    __builtin_memcpy(&r, &h, 2);
+    return r;
+}
+
+template <bool F16T>
+__device__ __forceinline__ uint16_t f32_to_t16(float x)
+{
+    if constexpr (F16T) return f32_to_f16_sat(x);
+    else return f32_to_bf16_rne(x);
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// decode kernel — the device form of read_array_compressed
+// ---------------------------------------------------------------------------
+// lut[q + bias] = fl((float)q / d) computed on the host in IEEE arithmetic, so the
+// strict result fl(lut * max) does not depend on the device's division.
+struct DecodeParams {
+    const uint8_t *codes;
+    float *out;
+    uint64_t n;
+    float max_val;       // scale from the file
+    float rel_scale;     // fl(max * fl(1/d))  (mode 1)
+    int mode;            // 0 strict, 1 release
+    float lut[256];
+};
+
+template <int FMT>
+__global__ __launch_bounds__(256) void sp_decode(const DecodeParams p)
+{
+    uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= p.n) return;
+    float v;
+    if constexpr (FMT == F32 || FMT == F16 || FMT == BF16) {
+        v = elem_value<FMT>(p.codes, i);
+    } else {
+        if (!(p.max_val > 0.0f)) {
+            v = 0.0f;
+        } else {
+            int q = int_code<FMT>(p.codes, i);
+            if (FMT == I2) v = __fmul_rn((float)q, p.max_val);                    // Serialize.c:285
+            else if (p.mode == 1) v = __fmul_rn((float)q, p.rel_scale);
+            else v = __fmul_rn(p.lut[q + (FMT == I8 ? 128 : 8)], p.max_val);      // Serialize.c:233,258
+        }
+    }
+    p.out[i] = v;
+}
+
+// ---------------------------------------------------------------------------
+// GEMV family (n <= 64): y[b][j] = act(bias[j] + scale * sum_k q[j][k] x[b][k])
+// ---------------------------------------------------------------------------
+struct LayerArgs {
+    const uint8_t *w;      // serialized weight codes, row-major [N][K]
+    const uint8_t *bias;   // serialized bias codes [N]
+    float wscale;          // folded weight scale
+    float bscale;          // folded bias scale
+    int bias_fmt;
+    int act;               // activation applied in the epilogue (A_NONE for softmax layers)
+    uint32_t N, K;         // out, in
+};
+
+// unpack one 16-byte chunk into its 128/bits unscaled float values
+template <int FMT>
+__device__ __forceinline__ void unpack16(const uint4 v, float *o)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (FMT == F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = bits_to_float(w[i]);
+    } else if constexpr (FMT == BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i]     = bits_to_float(w[i] << 16);
+            o[2 * i + 1] = bits_to_float(w[i] & 0xFFFF0000u);
+        }
+    } else if constexpr (FMT == F16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            _Float16 lo, hi;
+            uint16_t a = (uint16_t)(w[i] & 0xFFFFu), b = (uint16_t)(w[i] >> 16);
+            __builtin_memcpy(&lo, &a, 2);
+            __builtin_memcpy(&hi, &b, 2);
+            o[2 * i] = (float)lo;
+            o[2 * i + 1] = (float)hi;
+        }
+    } else if constexpr (FMT == I8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[4 * i + j] = (float)((int)(w[i] << (24 - 8 * j)) >> 24);
+    } else if constexpr (FMT == I4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[8 * i + j] = (float)((int)(w[i] << (28 - 4 * j)) >> 28);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[16 * i + j] = (float)((int)(w[i] << (30 - 2 * j)) >> 30);
+    }
+}
+
+// Aligned path: every row is a whole number of 16-byte chunks.  One wave owns
+// R rows at a time; lane c takes chunks c, c+64, ... of each row, so a wave reads
+// 1 KiB contiguous per row and instruction.  Partial sums meet in a
+// wavefront-shuffle reduction; lane 0 applies scale, bias and activation.
+template <int FMT, int BT, int R>
+__global__ __launch_bounds__(256) void sp_gemv(const LayerArgs L, const float *__restrict__ x,
+                                               float *__restrict__ y, int nb)
+{
+    constexpr int EPC = 128 / fmt_bits(FMT);
+    const int lane = threadIdx.x & 63;
+    const uint32_t wave = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t row0 = wave * R;
+    if (row0 >= L.N) return;
+    const uint32_t nchunks = L.K / EPC;
+    const size_t row_bytes = (size_t)nchunks * 16u;
+
+    const uint8_t *rp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        uint32_t row = row0 + r < L.N ? row0 + r : L.N - 1;
+        rp[r] = L.w + (size_t)row * row_bytes;
+    }
+
+    float acc[R][BT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[r][b] = 0.0f;
+
+    for (uint32_t c = lane; c < nchunks; c += kWave) {
+        uint4 wv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) wv[r] = *reinterpret_cast<const uint4 *>(rp[r] + (size_t)c * 16u);
+        float wf[R][EPC];
+#pragma unroll
+        for (int r = 0; r < R; ++r) unpack16<FMT>(wv[r], wf[r]);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const int bb = b < nb ? b : nb - 1;
+            const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)c * EPC);
+#pragma unroll
+            for (int e = 0; e < EPC / 4; ++e) {
+                float4 xv = xp[e];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    acc[r][b] = fmaf(wf[r][4 * e + 0], xv.x, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 1], xv.y, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 2], xv.z, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 3], xv.w, acc[r][b]);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[r][b] = wave_sum(acc[r][b]);
+
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = row0 + r;
+            if (row >= L.N) break;
+            const float bias = elem_value_rt(L.bias_fmt, L.bias, row) * L.bscale;
+#pragma unroll
+            for (int b = 0; b < BT; ++b)
+                if (b < nb) y[(size_t)b * L.N + row] = apply_act(fmaf(acc[r][b], L.wscale, bias), L.act);
+        }
+    }
+}
+
+// Generic path: any K, rows may start inside a byte.  One wave per row, one
+// element per lane and step.
+template <int FMT, int BT>
+__global__ __launch_bounds__(256) void sp_gemv_generic(const LayerArgs L, const float *__restrict__ x,
+                                                       float *__restrict__ y, int nb)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= L.N) return;
+    float acc[BT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+    const uint64_t base = (uint64_t)row * L.K;
+    for (uint32_t k = lane; k < L.K; k += kWave) {
+        const float w = elem_value<FMT>(L.w, base + k);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const int bb = b < nb ? b : nb - 1;
+            acc[b] = fmaf(w, x[(size_t)bb * L.K + k], acc[b]);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BT; ++b) acc[b] = wave_sum(acc[b]);
+    if (lane == 0) {
+        const float bias = elem_value_rt(L.bias_fmt, L.bias, row) * L.bscale;
+#pragma unroll
+        for (int b = 0; b < BT; ++b)
+            if (b < nb) y[(size_t)b * L.N + row] = apply_act(fmaf(acc[b], L.wscale, bias), L.act);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// softmax over rows (Activation.c:5-21); one wave per row
+// ---------------------------------------------------------------------------
+// out_kind: 0 FP32, 1 BF16, 2 FP16
+__global__ __launch_bounds__(256) void sp_softmax_rows(const float *__restrict__ in, void *__restrict__ out,
+                                                       int out_kind, uint32_t rows, uint32_t width)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *p = in + (size_t)row * width;
+    float m = -3.402823466e+38f;
+    for (uint32_t i = lane; i < width; i += kWave) m = fmaxf(m, p[i]);
+    m = wave_max(m);
+    float s = 0.0f;
+    for (uint32_t i = lane; i < width; i += kWave) s += expf(p[i] - m);
+    s = wave_sum(s);
+    const float inv = s > 0.0f ? 1.0f / s : 1.0f;
+    for (uint32_t i = lane; i < width; i += kWave) {
+        const float v = expf(p[i] - m) * inv;
+        const size_t o = (size_t)row * width + i;
+        if (out_kind == 0) reinterpret_cast<float *>(out)[o] = v;
+        else if (out_kind == 1) reinterpret_cast<uint16_t *>(out)[o] = f32_to_bf16_rne(v);
+        else reinterpret_cast<uint16_t *>(out)[o] = f32_to_f16_sat(v);
+    }
+}
+
+// FP32 -> 16-bit activations for the first GEMM layer
+template <bool F16T>
+__global__ __launch_bounds__(256) void sp_cvt16(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n)
+{
+    uint64_t i = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (i + 4 <= n) {
+        float4 v = *reinterpret_cast<const float4 *>(in + i);
+        uint2 o;
+        o.x = (uint32_t)f32_to_t16<F16T>(v.x) | ((uint32_t)f32_to_t16<F16T>(v.y) << 16);
+        o.y = (uint32_t)f32_to_t16<F16T>(v.z) | ((uint32_t)f32_to_t16<F16T>(v.w) << 16);
+        *reinterpret_cast<uint2 *>(out + i) = o;
+    } else {
+        for (; i < n; ++i) out[i] = f32_to_t16<F16T>(in[i]);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// 16-bit MFMA GEMM (n > 64): C[M][N] = act(bias + scale * A[M][K] . Wq[N][K]^T)
+// ---------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+struct GemmArgs {
+    LayerArgs L;
+    const uint16_t *A;     // [M][K] 16-bit activations
+    void *C;               // [M][N] 16-bit, or FP32 when out_f32
+    uint32_t M;
+    int out_f32;
+};
+
+// (float)q as a 16-bit float; exact for |q| <= 128 in either type
+template <bool F16T>
+__device__ __forceinline__ uint32_t int_to_t16(int q)
+{
+    if constexpr (F16T) {
+        _Float16 h = (_Float16)q;
+        uint16_t r;
+        __builtin_memcpy(&r, &h, 2);
+        return r;
+    } else {
+        return __float_as_uint((float)q) >> 16;
+    }
+}
+
+// unpack one 32-bit word of codes into 16-bit floats, written as packed pairs
+template <int FMT, bool F16T>
+__device__ __forceinline__ void unpack_word16(uint32_t w, uint32_t *o)
+{
+    constexpr int bits = fmt_bits(FMT);
+    constexpr int cnt = 32 / bits;
+#pragma unroll
+    for (int j = 0; j < cnt; j += 2) {
+        int q0 = (int)(w << (32 - bits - bits * j)) >> (32 - bits);
+        int q1 = (int)(w << (32 - bits - bits * (j + 1))) >> (32 - bits);
+        o[j / 2] = int_to_t16<F16T>(q0) | (int_to_t16<F16T>(q1) << 16);
+    }
+}
+
+// Tile: BM x BN x 64, 256 threads = 2 x 2 waves, each wave TM x TN tiles of 32x32.
+// LDS rows are padded by 8 elements so that 128-bit fragment reads of 32
+// consecutive rows spread over the banks.
+template <int FMT, bool F16T, int TM, int TN, bool ALIGNED>
+__global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
+{
+    constexpr int BM = 64 * TM, BN = 64 * TN, BK = 64, LDK = BK + 8;
+    constexpr int bits = fmt_bits(FMT);
+    constexpr int EPL = 128 / bits;                 // weight elements per 16-byte load
+    constexpr int W_LOADS = (BN * BK / EPL + 255) / 256;
+    constexpr int A_LOADS = BM * BK / 8 / 256;
+
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * LDK];
+
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // tile index: consecutive workgroups go to different XCDs, so give each XCD a
+    // contiguous band of tiles (shared A rows / W rows stay in one L2)
+    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = ntiles / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    const uint32_t tm = bid / tiles_n, tn = bid % tiles_n;
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    uint4 ra[A_LOADS], rw[W_LOADS];
+    const size_t w_row_bytes = (size_t)K * bits / 8u;
+
+    auto load_tiles = [&](uint32_t k0) {
+        if constexpr (ALIGNED) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+                const uint32_t k = k0 + kc * 8;
+                ra[i] = k < K ? *reinterpret_cast<const uint4 *>(g.A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + 256 * i;
+                constexpr int LPR = BK / EPL;           // loads per tile row
+                const int row = c / LPR, kc = c % LPR;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                const uint32_t k = k0 + kc * EPL;
+                const bool ok = (row < BN) && (k < K);
+                rw[i] = ok ? *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)k * bits / 8u)
+                           : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+
+    auto store_tiles = [&](uint32_t k0) {
+        if constexpr (ALIGNED) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                *reinterpret_cast<uint4 *>(&As[row * LDK + kc * 8]) = ra[i];
+            }
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + 256 * i;
+                constexpr int LPR = BK / EPL;
+                const int row = c / LPR, kc = c % LPR;
+                if (row >= BN) continue;
+                uint16_t *dst = &Ws[row * LDK + kc * EPL];
+                if constexpr (FMT == BF16 || FMT == F16) {
+                    *reinterpret_cast<uint4 *>(dst) = rw[i];
+                } else {
+                    const uint32_t w[4] = {rw[i].x, rw[i].y, rw[i].z, rw[i].w};
+                    constexpr int PW = 16 / bits;       // packed pairs per 32-bit word
+                    uint32_t o[4 * PW];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) unpack_word16<FMT, F16T>(w[q], o + q * PW);
+#pragma unroll
+                    for (int v = 0; v < PW; ++v)
+                        *reinterpret_cast<uint4 *>(dst + v * 8) = make_uint4(o[4 * v], o[4 * v + 1], o[4 * v + 2], o[4 * v + 3]);
+                }
+            }
+        } else {
+            // element-wise, fully bounds-checked
+            for (int e = t; e < BM * BK; e += 256) {
+                const int row = e / BK, kk = e % BK;
+                const uint32_t m = m0 + row, k = k0 + kk;
+                As[row * LDK + kk] = (m < M && k < K) ? g.A[(size_t)m * K + k] : (uint16_t)0;
+            }
+            for (int e = t; e < BN * BK; e += 256) {
+                const int row = e / BK, kk = e % BK;
+                const uint32_t n = n0 + row, k = k0 + kk;
+                uint16_t v = 0;
+                if (n < N && k < K) {
+                    const uint64_t idx = (uint64_t)n * K + k;
+                    if constexpr (FMT == BF16 || FMT == F16) v = reinterpret_cast<const uint16_t *>(g.L.w)[idx];
+                    else if constexpr (FMT == F32) v = f32_to_t16<F16T>(reinterpret_cast<const float *>(g.L.w)[idx]);
+                    else v = (uint16_t)int_to_t16<F16T>(int_code<FMT>(g.L.w, idx));
+                }
+                Ws[row * LDK + kk] = v;
+            }
+        }
+    };
+
+    const uint32_t ktiles = (K + BK - 1) / BK;
+    load_tiles(0);
+    for (uint32_t kt = 0; kt < ktiles; ++kt) {
+        __syncthreads();                              // previous tile fully consumed
+        store_tiles(kt * BK);
+        __syncthreads();
+        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
+
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            const int koff = ks + 8 * (lane >> 5);
+            uint4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[i] = *reinterpret_cast<const uint4 *>(&As[(wm * TM * 32 + i * 32 + (lane & 31)) * LDK + koff]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                fb[j] = *reinterpret_cast<const uint4 *>(&Ws[(wn * TN * 32 + j * 32 + (lane & 31)) * LDK + koff]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (F16T) {
+                        f16x8 a, b;
+                        __builtin_memcpy(&a, &fa[i], 16);
+                        __builtin_memcpy(&b, &fb[j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
+                    } else {
+                        bf16x8 a, b;
+                        __builtin_memcpy(&a, &fa[i], 16);
+                        __builtin_memcpy(&b, &fb[j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
+                    }
+                }
+        }
+    }
+
+    // epilogue: scale, bias, activation, store
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= M) continue;
+                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
+                const size_t o = (size_t)row * N + col;
+                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// FP32 MFMA GEMM for FP32 weights (n > 64): 64 x 64 x 16 tile, 4 waves
+// ---------------------------------------------------------------------------
+struct Gemm32Args {
+    LayerArgs L;
+    const float *A;
+    float *C;
+    uint32_t M;
+};
+
+__global__ __launch_bounds__(256) void sp_gemm32_f32(const Gemm32Args g)
+{
+    constexpr int BM = 64, BN = 64, BK = 16, LDK = BK + 1;
+    __shared__ float As[BM * LDK];
+    __shared__ float Ws[BN * LDK];
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t tiles_n = (N + BN - 1) / BN;
+    const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    const float *Wf = reinterpret_cast<const float *>(g.L.w);
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+    for (uint32_t k0 = 0; k0 < K; k0 += BK) {
+        __syncthreads();
+        for (int e = t; e < BM * BK; e += 256) {
+            const int row = e / BK, kk = e % BK;
+            const uint32_t m = m0 + row, n = n0 + row, k = k0 + kk;
+            As[row * LDK + kk] = (m < M && k < K) ? g.A[(size_t)m * K + k] : 0.0f;
+            Ws[row * LDK + kk] = (n < N && k < K) ? Wf[(size_t)n * K + k] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 2) {
+            const float a = As[(wm * 32 + (lane & 31)) * LDK + ks + (lane >> 5)];
+            const float b = Ws[(wn * 32 + (lane & 31)) * LDK + ks + (lane >> 5)];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        }
+    }
+
+    const uint32_t col = n0 + wn * 32 + (lane & 31);
+    if (col >= N) return;
+    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < M) g.C[(size_t)row * N + col] = apply_act(acc[r] + bias, g.L.act);
+    }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct DevArray {
+    uint8_t *base = nullptr;       // allocation (256-byte aligned by hipMalloc)
+    size_t bytes = 0;
+    uint64_t count = 0;
+    float max_val = 0.0f;
+    bool uploaded = false;
+};
+
+struct sphip_net {
+    uint32_t layers = 0;
+    std::vector<uint32_t> topo;
+    std::vector<uint8_t> act;
+    int prec = 0;
+    std::vector<DevArray> W, B;    // [layers-1]
+    // workspace, grown on demand
+    uint64_t cap_elems = 0;        // capacity of each ping-pong buffer in FP32 elements
+    void *buf[2] = {nullptr, nullptr};
+    float *soft_tmp = nullptr;     // FP32 logits of a softmax layer
+    uint64_t soft_cap = 0;
+    float *layers_buf = nullptr;   // per-layer activations of a KEEP_LAYERS forward
+    float *stage_x = nullptr;      // device staging of host inputs / outputs
+    float *stage_y = nullptr;
+    uint64_t stage_x_cap = 0, stage_y_cap = 0;
+    uint32_t max_width = 0;
+    uint64_t total_neurons = 0;
+};
+
+namespace {
+
+enum Regime { R_GEMV, R_GEMM16, R_GEMM32 };
+
+Regime pick_regime(const sphip_net *net, uint32_t n, uint32_t flags)
+{
+    if ((flags & SPHIP_FORCE_GEMV) && n <= 64) return R_GEMV;
+    if (flags & SPHIP_FORCE_GEMM) return net->prec == F32 ? R_GEMM32 : R_GEMM16;
+    if (n <= 64) return R_GEMV;
+    return net->prec == F32 ? R_GEMM32 : R_GEMM16;
+}
+
+LayerArgs make_layer_args(const sphip_net *net, uint32_t l /*1-based layer*/)
+{
+    LayerArgs L{};
+    const DevArray &w = net->W[l - 1], &b = net->B[l - 1];
+    L.w = w.base;
+    L.bias = b.base;
+    L.wscale = fmt_scale(net->prec, w.max_val);
+    L.bscale = fmt_scale(net->prec, b.max_val);
+    L.bias_fmt = net->prec;
+    L.act = net->act[l - 1] == A_SOFTMAX ? A_NONE : net->act[l - 1];
+    L.N = net->topo[l];
+    L.K = net->topo[l - 1];
+    return L;
+}
+
+bool rows_aligned(int fmt, uint32_t K) { return ((uint64_t)K * (uint64_t)fmt_bits(fmt)) % 128u == 0; }
+
+template <int FMT>
+void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
+{
+    const bool aligned = rows_aligned(FMT, L.K) && (L.K % 4u == 0);
+    for (uint32_t b0 = 0; b0 < n; b0 += 8) {
+        const int nb = (int)(n - b0 < 8 ? n - b0 : 8);
+        const float *xb = x + (size_t)b0 * L.K;
+        float *yb = y + (size_t)b0 * L.N;
+        if (aligned) {
+            constexpr int R = 2;
+            const uint32_t waves = (L.N + R - 1) / R, grid = (waves + 3) / 4;
+            if (nb == 1) sp_gemv<FMT, 1, R><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+            else if (nb == 2) sp_gemv<FMT, 2, R><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+            else if (nb <= 4) sp_gemv<FMT, 4, R><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+            else sp_gemv<FMT, 8, R><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+        } else {
+            const uint32_t grid = (L.N + 3) / 4;
+            if (nb == 1) sp_gemv_generic<FMT, 1><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+            else if (nb <= 4) sp_gemv_generic<FMT, 4><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+            else sp_gemv_generic<FMT, 8><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb);
+        }
+    }
+}
+
+void launch_gemv(int fmt, const LayerArgs &L, const float *x, float *y, uint32_t n)
+{
+    switch (fmt) {
+    case F32:  launch_gemv_fmt<F32>(L, x, y, n); break;
+    case F16:  launch_gemv_fmt<F16>(L, x, y, n); break;
+    case BF16: launch_gemv_fmt<BF16>(L, x, y, n); break;
+    case I8:   launch_gemv_fmt<I8>(L, x, y, n); break;
+    case I4:   launch_gemv_fmt<I4>(L, x, y, n); break;
+    default:   launch_gemv_fmt<I2>(L, x, y, n); break;
+    }
+}
+
+template <int FMT, bool F16T>
+void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
+{
+    GemmArgs g{L, A, C, M, out_f32};
+    constexpr int TM = 2, TN = 2, BM = 64 * TM, BN = 64 * TN;
+    const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
+    const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
+    if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
+    else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
+}
+
+void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
+{
+    switch (fmt) {
+    case F16:  launch_gemm16_fmt<F16, true>(L, A, C, M, out_f32); break;
+    case BF16: launch_gemm16_fmt<BF16, false>(L, A, C, M, out_f32); break;
+    case I8:   launch_gemm16_fmt<I8, false>(L, A, C, M, out_f32); break;
+    case I4:   launch_gemm16_fmt<I4, false>(L, A, C, M, out_f32); break;
+    default:   launch_gemm16_fmt<I2, false>(L, A, C, M, out_f32); break;    // FP32 weights never come here
+    }
+}
+
+void launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M)
+{
+    Gemm32Args g{L, A, C, M};
+    const uint32_t grid = ((M + 63) / 64) * ((L.N + 63) / 64);
+    sp_gemm32_f32<<<grid, 256, 0, g_stream>>>(g);
+}
+
+int reserve(sphip_net *net, uint32_t n, bool keep_layers)
+{
+    const uint64_t need = (uint64_t)n * net->max_width;
+    if (need > net->cap_elems) {
+        for (int i = 0; i < 2; ++i) {
+            if (net->buf[i]) { HCHECK(hipFree(net->buf[i])); net->buf[i] = nullptr; }
+        }
+        net->cap_elems = 0;
+        for (int i = 0; i < 2; ++i) HCHECK(hipMalloc(&net->buf[i], need * sizeof(float)));
+        net->cap_elems = need;
+    }
+    uint64_t soft = 0;
+    for (uint32_t l = 1; l < net->layers; ++l)
+        if (net->act[l - 1] == A_SOFTMAX && (uint64_t)n * net->topo[l] > soft) soft = (uint64_t)n * net->topo[l];
+    if (soft > net->soft_cap) {
+        if (net->soft_tmp) { HCHECK(hipFree(net->soft_tmp)); net->soft_tmp = nullptr; }
+        net->soft_cap = 0;
+        HCHECK(hipMalloc((void **)&net->soft_tmp, soft * sizeof(float)));
+        net->soft_cap = soft;
+    }
+    if (keep_layers && !net->layers_buf)
+        HCHECK(hipMalloc((void **)&net->layers_buf, net->total_neurons * sizeof(float)));
+    return 0;
+}
+
+int grow(float **p, uint64_t *cap, uint64_t need)
+{
+    if (need <= *cap) return 0;
+    if (*p) { HCHECK(hipFree(*p)); *p = nullptr; }
+    *cap = 0;
+    HCHECK(hipMalloc((void **)p, need * sizeof(float)));
+    *cap = need;
+    return 0;
+}
+
+int check_uploaded(const sphip_net *net)
+{
+    for (uint32_t l = 0; l + 1 < net->layers; ++l)
+        if (!net->W[l].uploaded || !net->B[l].uploaded) return fail_msg("sphip: an array of this net was never uploaded");
+    return 0;
+}
+
+// Enqueues every kernel of one forward.  d_x, d_y are device pointers.
+// only_layer != 0 restricts the launch to the main kernel of that layer.
+int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags, uint32_t only_layer)
+{
+    const bool keep = (flags & SPHIP_KEEP_LAYERS) != 0;
+    const Regime reg = pick_regime(net, n, flags);
+    const bool f16t = net->prec == F16;
+    const uint32_t last = net->layers - 1;
+
+    const void *in = d_x;
+    if (reg == R_GEMM16 && !only_layer) {
+        const uint64_t cnt = (uint64_t)n * net->topo[0];
+        const uint32_t grid = (uint32_t)((cnt / 4 + 255) / 256 + 1);
+        if (f16t) sp_cvt16<true><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)net->buf[1], cnt);
+        else sp_cvt16<false><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)net->buf[1], cnt);
+        in = net->buf[1];
+    } else if (reg == R_GEMM16) {
+        in = net->buf[1];
+    }
+    if (keep)
+        HCHECK(hipMemcpyAsync(net->layers_buf, d_x, (size_t)net->topo[0] * sizeof(float), hipMemcpyDeviceToDevice, g_stream));
+
+    uint64_t noff = net->topo[0];
+    for (uint32_t l = 1; l <= last; ++l) {
+        const LayerArgs L = make_layer_args(net, l);
+        const bool softmax = net->act[l - 1] == A_SOFTMAX;
+        const bool is_last = l == last;
+        void *dst = is_last ? (void *)d_y : net->buf[(l + 1) & 1];
+        // logits of a softmax layer go to FP32 scratch first
+        void *main_out = softmax ? (void *)net->soft_tmp : dst;
+        const int out_f32 = (reg != R_GEMM16) || is_last || softmax;
+        const bool run = !only_layer || only_layer == l;
+        if (run) {
+            if (reg == R_GEMV) launch_gemv(net->prec, L, (const float *)in, (float *)main_out, n);
+            else if (reg == R_GEMM32) launch_gemm32(L, (const float *)in, (float *)main_out, n);
+            else launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32);
+        }
+        if (softmax && !only_layer) {
+            const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
+            sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(net->soft_tmp, dst, kind, n, net->topo[l]);
+        }
+        if (keep)     // n == 1 and FP32 activations: mirror the layer into the neurons-shaped buffer
+            HCHECK(hipMemcpyAsync(net->layers_buf + noff, dst, (size_t)net->topo[l] * sizeof(float),
+                                  hipMemcpyDeviceToDevice, g_stream));
+        in = dst;
+        noff += net->topo[l];
+    }
+    HCHECK(hipGetLastError());
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sphip_device_count(void)
+{
+    int cnt = 0;
+    if (hipGetDeviceCount(&cnt) != hipSuccess) return 0;
+    return cnt;
+}
+
+const char *sphip_last_error_string(void) { return g_err; }
+
+int sphip_create(const sphip_desc *desc, sphip_net **out)
+{
+    if (!desc || !out || desc->layers < 2 || !desc->topology || !desc->act) return fail_msg("sphip_create: invalid descriptor");
+    if (desc->precision >= NFMT) return fail_msg("sphip_create: invalid precision");
+    for (uint32_t l = 0; l < desc->layers; ++l)
+        if (desc->topology[l] == 0) return fail_msg("sphip_create: empty layer");
+    for (uint32_t l = 0; l + 1 < desc->layers; ++l)
+        if (desc->act[l] >= A_COUNT) return fail_msg("sphip_create: invalid activation");
+    if (ensure_stream()) return 1;
+    sphip_net *net = new (std::nothrow) sphip_net;
+    if (!net) return fail_msg("sphip_create: out of host memory");
+    net->layers = desc->layers;
+    net->topo.assign(desc->topology, desc->topology + desc->layers);
+    net->act.assign(desc->act, desc->act + desc->layers - 1);
+    net->prec = desc->precision;
+    net->W.resize(desc->layers - 1);
+    net->B.resize(desc->layers - 1);
+    for (uint32_t l = 0; l < desc->layers; ++l) {
+        if (net->topo[l] > net->max_width) net->max_width = net->topo[l];
+        net->total_neurons += net->topo[l];
+    }
+    for (uint32_t l = 0; l + 1 < desc->layers; ++l) {
+        DevArray &w = net->W[l], &b = net->B[l];
+        w.count = (uint64_t)net->topo[l] * net->topo[l + 1];
+        b.count = net->topo[l + 1];
+        w.bytes = fmt_bytes(net->prec, w.count);
+        b.bytes = fmt_bytes(net->prec, b.count);
+        // 16 bytes of slack: vector loads of the last chunk never leave the allocation
+        if (hipMalloc((void **)&w.base, w.bytes + 16) != hipSuccess || hipMalloc((void **)&b.base, b.bytes + 16) != hipSuccess) {
+            sphip_destroy(net);
+            return fail_msg("sphip_create: device allocation failed");
+        }
+    }
+    *out = net;
+    return 0;
+}
+
+void sphip_destroy(sphip_net *net)
+{
+    if (!net) return;
+    if (g_stream) (void)hipStreamSynchronize(g_stream);
+    for (auto &a : net->W) if (a.base) (void)hipFree(a.base);
+    for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
+    for (int i = 0; i < 2; ++i) if (net->buf[i]) (void)hipFree(net->buf[i]);
+    if (net->soft_tmp) (void)hipFree(net->soft_tmp);
+    if (net->layers_buf) (void)hipFree(net->layers_buf);
+    if (net->stage_x) (void)hipFree(net->stage_x);
+    if (net->stage_y) (void)hipFree(net->stage_y);
+    delete net;
+}
+
+int sphip_upload_array(sphip_net *net, uint32_t l, int which, const void *codes, size_t bytes, float max_val)
+{
+    if (!net || l + 1 >= net->layers || (which != 0 && which != 1) || !codes) return fail_msg("sphip_upload_array: invalid argument");
+    DevArray &a = which == 0 ? net->W[l] : net->B[l];
+    if (bytes != a.bytes) return fail_msg("sphip_upload_array: byte count does not match the array's serialized size");
+    HCHECK(hipMemcpyAsync(a.base, codes, bytes, hipMemcpyHostToDevice, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    a.max_val = max_val;
+    a.uploaded = true;
+    return 0;
+}
+
+int sphip_clone(const sphip_net *src, sphip_net **out)
+{
+    if (!src || !out) return fail_msg("sphip_clone: invalid argument");
+    sphip_desc d{src->layers, src->topo.data(), src->act.data(), (uint8_t)src->prec};
+    sphip_net *net = nullptr;
+    if (sphip_create(&d, &net)) return 1;
+    for (uint32_t l = 0; l + 1 < src->layers; ++l) {
+        for (int which = 0; which < 2; ++which) {
+            const DevArray &s = which == 0 ? src->W[l] : src->B[l];
+            DevArray &t = which == 0 ? net->W[l] : net->B[l];
+            hipError_t e = hipMemcpyAsync(t.base, s.base, s.bytes, hipMemcpyDeviceToDevice, g_stream);
+            if (e != hipSuccess) { sphip_destroy(net); return fail_hip("sphip_clone copy", e); }
+            t.max_val = s.max_val;
+            t.uploaded = s.uploaded;
+        }
+    }
+    HCHECK(hipStreamSynchronize(g_stream));
+    *out = net;
+    return 0;
+}
+
+int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t flags)
+{
+    if (!net || !x || !y || n == 0) return fail_msg("sphip_forward: invalid argument");
+    if ((flags & SPHIP_KEEP_LAYERS) && n != 1) return fail_msg("sphip_forward: SPHIP_KEEP_LAYERS needs n == 1");
+    if (check_uploaded(net)) return 1;
+    if (reserve(net, n, (flags & SPHIP_KEEP_LAYERS) != 0)) return 1;
+    const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * net->topo[net->layers - 1];
+    const float *d_x = x;
+    float *d_y = y;
+    if (!(flags & SPHIP_X_ON_DEVICE)) {
+        if (grow(&net->stage_x, &net->stage_x_cap, in_cnt)) return 1;
+        HCHECK(hipMemcpyAsync(net->stage_x, x, in_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        d_x = net->stage_x;
+    }
+    if (!(flags & SPHIP_Y_ON_DEVICE)) {
+        if (grow(&net->stage_y, &net->stage_y_cap, out_cnt)) return 1;
+        d_y = net->stage_y;
+    }
+    if (enqueue_forward(net, d_x, n, d_y, flags, 0)) return 1;
+    if (!(flags & SPHIP_Y_ON_DEVICE)) {
+        HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
+        HCHECK(hipStreamSynchronize(g_stream));
+    }
+    return 0;
+}
+
+int sphip_read_layers(sphip_net *net, float *host_neurons)
+{
+    if (!net || !host_neurons || !net->layers_buf) return fail_msg("sphip_read_layers: no kept activations");
+    HCHECK(hipMemcpyAsync(host_neurons, net->layers_buf, net->total_neurons * sizeof(float), hipMemcpyDeviceToHost, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int sphip_decode(sphip_net *net, uint32_t l, int which, int mode, float *host_out)
+{
+    if (!net || l + 1 >= net->layers || (which != 0 && which != 1) || !host_out || (mode != 0 && mode != 1))
+        return fail_msg("sphip_decode: invalid argument");
+    const DevArray &a = which == 0 ? net->W[l] : net->B[l];
+    if (!a.uploaded) return fail_msg("sphip_decode: array not uploaded");
+    float *d_out = nullptr;
+    HCHECK(hipMalloc((void **)&d_out, a.count * sizeof(float)));
+    DecodeParams p{};
+    p.codes = a.base;
+    p.out = d_out;
+    p.n = a.count;
+    p.max_val = a.max_val;
+    p.mode = mode;
+    const float d = fmt_divisor(net->prec);
+    {
+        volatile float r = 1.0f / d;
+        volatile float s = a.max_val * r;
+        p.rel_scale = s;
+    }
+    if (net->prec == I8) for (int q = -128; q < 128; ++q) { volatile float fq = (float)q; volatile float tq = fq / 127.0f; p.lut[q + 128] = tq; }
+    if (net->prec == I4) for (int q = -8; q < 8; ++q) { volatile float fq = (float)q; volatile float tq = fq / 7.0f; p.lut[q + 8] = tq; }
+    const uint32_t grid = (uint32_t)((a.count + 255) / 256);
+    switch (net->prec) {
+    case F32:  sp_decode<F32><<<grid, 256, 0, g_stream>>>(p); break;
+    case F16:  sp_decode<F16><<<grid, 256, 0, g_stream>>>(p); break;
+    case BF16: sp_decode<BF16><<<grid, 256, 0, g_stream>>>(p); break;
+    case I8:   sp_decode<I8><<<grid, 256, 0, g_stream>>>(p); break;
+    case I4:   sp_decode<I4><<<grid, 256, 0, g_stream>>>(p); break;
+    default:   sp_decode<I2><<<grid, 256, 0, g_stream>>>(p); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpyAsync(host_out, d_out, a.count * sizeof(float), hipMemcpyDeviceToHost, g_stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_stream);
+    (void)hipFree(d_out);
+    if (e != hipSuccess) return fail_hip("sphip_decode", e);
+    return 0;
+}
+
+int sphip_synchronize(void)
+{
+    if (!g_stream) return 0;
+    HCHECK(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int sphip_malloc(void **dptr, size_t bytes)
+{
+    if (!dptr) return fail_msg("sphip_malloc: null");
+    if (ensure_stream()) return 1;
+    HCHECK(hipMalloc(dptr, bytes ? bytes : 1));
+    return 0;
+}
+
+int sphip_free(void *dptr)
+{
+    if (dptr) HCHECK(hipFree(dptr));
+    return 0;
+}
+
+int sphip_memcpy_h2d(void *dst, const void *src, size_t bytes)
+{
+    if (ensure_stream()) return 1;
+    HCHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+int sphip_memcpy_d2h(void *dst, const void *src, size_t bytes)
+{
+    if (ensure_stream()) return 1;
+    HCHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
+static int time_common(sphip_net *const *nets, int count, const float *d_x, uint32_t n, float *d_y,
+                       uint32_t flags, int iters, float *ms, uint32_t only_layer)
+{
+    if (!nets || count <= 0 || iters <= 0 || !ms) return fail_msg("sphip_time: invalid argument");
+    for (int i = 0; i < count; ++i) {
+        if (!nets[i]) return fail_msg("sphip_time: null net");
+        if (check_uploaded(nets[i])) return 1;
+        if (reserve(nets[i], n, false)) return 1;
+    }
+    hipEvent_t e0, e1;
+    HCHECK(hipEventCreate(&e0));
+    HCHECK(hipEventCreate(&e1));
+    int rc = 0;
+    HCHECK(hipEventRecord(e0, g_stream));
+    for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward(nets[it % count], d_x, n, d_y, flags, only_layer);
+    hipError_t e = hipEventRecord(e1, g_stream);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail_hip("sphip_time", e);
+    return 0;
+}
+
+int sphip_time_forward(sphip_net *const *nets, int count, const float *d_x, uint32_t n, float *d_y,
+                       uint32_t flags, int iters, float *ms)
+{
+    if (!d_x || !d_y || n == 0) return fail_msg("sphip_time_forward: invalid argument");
+    return time_common(nets, count, d_x, n, d_y, flags & ~SPHIP_KEEP_LAYERS, iters, ms, 0);
+}
+
+int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t n, uint32_t flags,
+                     int iters, float *ms)
+{
+    if (!nets || count <= 0 || !nets[0] || layer == 0 || layer >= nets[0]->layers || n == 0)
+        return fail_msg("sphip_time_layer: invalid argument");
+    // inputs and outputs are the nets' own scratch buffers (contents irrelevant for timing)
+    for (int i = 0; i < count; ++i) {
+        if (reserve(nets[i], n, false)) return 1;
+        if (grow(&nets[i]->stage_y, &nets[i]->stage_y_cap, (uint64_t)n * nets[i]->topo[nets[i]->layers - 1])) return 1;
+        if (grow(&nets[i]->stage_x, &nets[i]->stage_x_cap, (uint64_t)n * nets[i]->topo[0])) return 1;
+    }
+    return time_common(nets, count, nets[0]->stage_x, n, nets[0]->stage_y, flags & ~SPHIP_KEEP_LAYERS, iters, ms, layer);
+}
+
+const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, uint32_t flags)
+{
+    if (!net || layer == 0 || layer >= net->layers) return "";
+    switch (pick_regime(net, n, flags)) {
+    case R_GEMV:   return "sp_gemv";
+    case R_GEMM32: return "sp_gemm32_f32";
+    default:       return "sp_gemm16";
+    }
+}
+
+}  // extern "C"
