@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X inference forward pass.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+
+A step is one forward of one batch of seeded synthetic inputs through a net
+whose weights were written by the library's own serializer and loaded back
+(load_spingalett keeps the packed arrays; the device computes on them).
+Inputs and outputs are device-resident during the timed region.  One JSON line
+is printed: the headline workload plus, under "workloads", the other
+BASELINE configurations with their own roofline figures.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import spingalett_amd as S  # noqa: E402
+
+HBM_PEAK = 8.0e12          # B/s
+MFMA16_PEAK = 2.5e15       # FLOP/s, dense bf16/fp16
+FP32_PEAK = 157.3e12
+
+PREC_NAMES = {S.PRECISION_FLOAT32: "fp32", S.PRECISION_FP16: "fp16", S.PRECISION_BFLOAT16: "bf16",
+              S.PRECISION_INT8: "int8", S.PRECISION_INT4: "int4", S.PRECISION_INT2: "int2"}
+BITS = {S.PRECISION_FLOAT32: 32, S.PRECISION_FP16: 16, S.PRECISION_BFLOAT16: 16,
+        S.PRECISION_INT8: 8, S.PRECISION_INT4: 4, S.PRECISION_INT2: 2}
+
+A = dict(sigmoid=S.ACT_SIGMOID, relu=S.ACT_RELU, tanh=S.ACT_TANH, leaky=S.ACT_LEAKY_RELU,
+         foo52=S.ACT_FOO52, softmax=S.ACT_SOFTMAX, none=S.ACT_NONE)
+
+# name -> (topology, activations, init per layer, precision, input distribution, batches, headline batch)
+WORKLOADS = {
+    "C1": dict(topo=[784, 512, 1000, 10], acts=["relu", "relu", "softmax"], init=["he", "he", "xavier"],
+               prec=S.PRECISION_FLOAT32, inputs="u01", batches=[256]),
+    "C2": dict(topo=[784, 512, 1000, 10], acts=["relu", "relu", "softmax"], init=["he", "he", "xavier"],
+               prec=S.PRECISION_INT8, inputs="u01", batches=[1, 256, 4096]),
+    "C3": dict(topo=[4096, 16384, 16384, 4096], acts=["relu", "tanh", "none"], init=["xavier"] * 3,
+               prec=S.PRECISION_INT4, inputs="n01", batches=[1, 8, 64]),
+    "C4": dict(topo=[8192] * 9 + [1000], acts=["leaky", "foo52"] * 4 + ["softmax"], init=["he"] * 9,
+               prec=S.PRECISION_BFLOAT16, inputs="n01", batches=[8192]),
+    "C5": dict(topo=[2048, 8192, 8192, 8192, 8192, 1000], acts=["sigmoid", "relu", "relu", "tanh", "softmax"],
+               init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1, 64, 4096, 65536]),
+}
+
+
+def array_payload(n: int, prec: int) -> int:
+    """Serialized size of an n-element array including its 4-byte scale (Serialize.c:87-193)."""
+    if prec == S.PRECISION_FLOAT32:
+        return 4 * n
+    if prec in (S.PRECISION_FP16, S.PRECISION_BFLOAT16):
+        return 2 * n
+    return 4 + (n * BITS[prec] + 7) // 8
+
+
+def algorithmic_bytes(topo, prec, batch) -> int:
+    w = sum(array_payload(topo[l] * topo[l + 1], prec) + array_payload(topo[l + 1], prec) for l in range(len(topo) - 1))
+    return w + 4 * batch * (topo[0] + topo[-1])
+
+
+def flops_per_sample(topo) -> int:
+    return 2 * sum(topo[l] * topo[l + 1] for l in range(len(topo) - 1))
+
+
+def build_net(name: str, seed: int = 42):
+    """Seeded FP32 net -> library writer -> file -> load_spingalett.  Returns (net, file path)."""
+    cfg = WORKLOADS[name]
+    topo, acts = cfg["topo"], cfg["acts"]
+    rng = np.random.default_rng(seed)
+    net = S.new_spingalett(S.LOSS_CROSS_ENTROPY)
+    S.layer(net, topo[0])
+    for l in range(1, len(topo)):
+        S.layer(net, topo[l], A[acts[l - 1]], S.WEIGHT_INITIALIZATION_NONE)
+    for l in range(len(topo) - 1):
+        std = np.float32(np.sqrt((2.0 if cfg["init"][l] == "he" else 1.0) / topo[l]))
+        W = S.weights_view(net, l)
+        # generated row block by row block to bound temporary memory
+        step = max(1, (1 << 26) // topo[l])
+        for r0 in range(0, topo[l + 1], step):
+            r1 = min(topo[l + 1], r0 + step)
+            W[r0:r1] = rng.standard_normal((r1 - r0, topo[l]), dtype=np.float32) * std
+        S.biases_view(net, l)[:] = rng.standard_normal(topo[l + 1], dtype=np.float32) * np.float32(0.05)
+    tmpdir = tempfile.mkdtemp(prefix="spbench_")
+    path = os.path.join(tmpdir, name + ".nn")
+    S.clear_error()
+    S.save_spingalett(net, path, cfg["prec"], do_not_save_optimizer=True)
+    code, msg = S.last_error()
+    if code:
+        raise RuntimeError("save_spingalett: " + msg)
+    S.free_network(net)
+    loaded = S.load_spingalett(path)
+    if loaded is None:
+        raise RuntimeError("load_spingalett: " + S.last_error()[1])
+    return loaded, path
+
+
+def make_inputs(kind: str, n: int, width: int, seed: int = 7) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    if kind == "u01":
+        return rng.random((n, width), dtype=np.float32)
+    if kind == "u11":
+        return rng.random((n, width), dtype=np.float32) * np.float32(2) - np.float32(1)
+    return rng.standard_normal((n, width), dtype=np.float32)
+
+
+class DevNetRef:
+    """Borrowed kernel-TU handle of a loaded net (so timing helpers can take it)."""
+    def __init__(self, handle):
+        self.h = C.c_void_p(handle)
+
+
+def device_copies(net, topo, prec, min_total_bytes: int):
+    """The net's own device copy plus clones until the rotation exceeds the last-level cache."""
+    h = S.lib().spingalett_hip_handle(net)
+    if not h:
+        raise RuntimeError("hip handle: " + S.last_error()[1])
+    base = DevNetRef(h)
+    nbytes = algorithmic_bytes(topo, prec, 0)
+    copies = [base]
+    clones = []
+    while nbytes * len(copies) < min_total_bytes:
+        hc = C.c_void_p()
+        if S.lib().sphip_clone(base.h, C.byref(hc)):
+            raise RuntimeError("sphip_clone: " + S.lib().sphip_last_error_string().decode())
+        clones.append(hc)
+        copies.append(DevNetRef(hc.value))
+    return copies, clones
+
+
+def time_workload(copies, topo, n, x_host, steps, warmup):
+    d_x = S.DeviceBuffer.from_numpy(x_host)
+    d_y = S.DeviceBuffer(4 * n * topo[-1])
+    if warmup > 0:
+        S.time_forward(copies, d_x, n, d_y, warmup)
+    S.synchronize()
+    t0 = time.perf_counter()
+    ev_ms = S.time_forward(copies, d_x, n, d_y, steps)      # records events, waits for the last one
+    S.synchronize()
+    wall = time.perf_counter() - t0
+    y = d_y.to_numpy(np.float32, (n, topo[-1]))
+    d_x.free()
+    d_y.free()
+    return wall * 1e3 / steps, ev_ms / steps, y
+
+
+def dominant_layer(topo):
+    return 1 + int(np.argmax([topo[l] * topo[l + 1] for l in range(len(topo) - 1)]))
+
+
+def roofline_for(copies, topo, prec, n, iters):
+    """Times the main kernel of the largest layer alone (HIP events on its stream)."""
+    l = dominant_layer(topo)
+    S.time_layer(copies, l, n, 2)
+    ms = S.time_layer(copies, l, n, iters) / iters
+    K, N = topo[l - 1], topo[l]
+    kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
+    if n <= 64:
+        # memory regime: serialized weights + bias of the layer, FP32 inputs and outputs of the layer
+        nbytes = array_payload(K * N, prec) + array_payload(N, prec) + 4 * n * (K + N)
+        ach = nbytes / (ms * 1e-3)
+        return dict(bound="hbm", achieved=ach / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s", frac=ach / HBM_PEAK,
+                    traffic=None, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+    fl = 2.0 * n * K * N
+    ach = fl / (ms * 1e-3)
+    peak = FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK
+    return dict(bound="mfma", achieved=ach / 1e12, peak=peak / 1e12, unit="TFLOP/s", frac=ach / peak,
+                traffic=None, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+
+
+def cpu_baseline(path, cfg, n_sample, budget_s=12.0):
+    """The reference's batched call sequence (sgemm NT + bias + activation,
+    Training.c:327-343) restated on the host, threaded BLAS, on a sample of the batch."""
+    import oracle as O
+    with open(path, "rb") as f:
+        blob = f.read()
+    net = O.Net.parse(blob)
+    del blob
+    sgemm, desc, set_threads = O.find_sgemm()
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    if set_threads is not None:
+        set_threads(cores)
+    X = make_inputs(cfg["inputs"], n_sample, cfg["topo"][0], seed=11)
+    sec, _ = net.time_forward_batch(X, 1, sgemm, cores)
+    iters = int(max(1, min(200, budget_s / max(sec, 1e-6))))
+    sec, _ = net.time_forward_batch(X, iters, sgemm, cores)
+    return dict(value=n_sample / sec, unit="samples/s", cores=cores, kind="port",
+                sample=f"{n_sample} samples x {iters} iterations of the same net on host cores, {desc}")
+
+
+def run_workload(name, batches, steps, warmup, want_output=False):
+    cfg = WORKLOADS[name]
+    topo, prec = cfg["topo"], cfg["prec"]
+    t0 = time.perf_counter()
+    net, path = build_net(name)
+    build_s = time.perf_counter() - t0
+    copies, clones = device_copies(net, topo, prec, 600 << 20 if algorithmic_bytes(topo, prec, 0) > (8 << 20) else 0)
+    rows = []
+    for n in batches:
+        x = make_inputs(cfg["inputs"], n, topo[0])
+        k = steps if n * flops_per_sample(topo) < 2e12 else max(3, min(steps, 20))
+        ms_wall, ms_ev, y = time_workload(copies, topo, n, x, k, warmup)
+        fl = flops_per_sample(topo) * n
+        row = dict(workload=name, format=PREC_NAMES[prec], batch=n, steps=k, ms_per_step=ms_wall, ms_per_step_events=ms_ev,
+                   samples_per_s=n / (ms_wall * 1e-3),
+                   hbm_frac=algorithmic_bytes(topo, prec, n) / (ms_ev * 1e-3) / HBM_PEAK,
+                   mfma_frac=fl / (ms_ev * 1e-3) / (FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK),
+                   copies=len(copies), finite=bool(np.isfinite(y).all()))
+        row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
+        rows.append(row)
+    return dict(net=net, path=path, copies=copies, clones=clones, rows=rows, build_s=build_s)
+
+
+def release(w):
+    for hc in w["clones"]:
+        S.lib().sphip_destroy(hc)
+    S.free_network(w["net"])
+    try:
+        os.remove(w["path"])
+        os.rmdir(os.path.dirname(w["path"]))
+    except OSError:
+        pass
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C4", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        return 2
+    S.set_verbose(False)
+    if S.device_count() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+
+    cfg = WORKLOADS[args.workload]
+    n = args.batch or max(cfg["batches"])
+    head = run_workload(args.workload, [n], args.steps, args.warmup)
+    row = head["rows"][0]
+    cpu = None
+    if not args.no_cpu:
+        sample = min(n, 512 if flops_per_sample(cfg["topo"]) > 5e8 else 4096)
+        cpu = cpu_baseline(head["path"], cfg, sample)
+    release(head)
+
+    extra = []
+    if not args.no_extra:
+        for name in ("C2", "C3", "C5", "C1"):
+            if name == args.workload:
+                continue
+            try:
+                w = run_workload(name, WORKLOADS[name]["batches"], 50, 3)
+                extra += w["rows"]
+                release(w)
+            except Exception as e:  # keep the headline even if an extra configuration fails
+                extra.append(dict(workload=name, error=str(e)))
+
+    rl = dict(row["roofline"])
+    out = {
+        "metric": "forward samples/sec per weight format; % peak HBM BW (b=1), % MFMA peak (b>=4K)",
+        "value": row["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": row["steps"], "warmup": args.warmup,
+        "ms_per_step": row["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"bf16": "bf16", "fp16": "f16", "fp32": "f32"}.get(row["format"], "bf16"),
+        "data": "synthetic (seeded normal weights through the library's serializer, seeded inputs)",
+        "config": {"workload": f"{args.workload}: {'->'.join(map(str, cfg['topo']))} {row['format']} weights, batch {n}",
+                   "format": row["format"], "batch": n},
+        "roofline": {k: rl[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "roofline_kernel": {k: rl[k] for k in ("kernel", "layer", "shape", "avg_ms")},
+        "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
+        "cpu_baseline": cpu,
+        "workloads": extra,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
