@@ -249,7 +249,8 @@ def forward_batch(net, X):
 
 
 def save_spingalett(net, filename: str, precision: int = PRECISION_FLOAT32, do_not_save_optimizer: bool = False):
-    lib().save_spingalett_struct_arguments(SaveArgs(net, os.fsencode(filename), do_not_save_optimizer, precision))
+    fn = None if filename is None else os.fsencode(filename)
+    lib().save_spingalett_struct_arguments(SaveArgs(net, fn, do_not_save_optimizer, precision))
 
 
 def load_spingalett(filename):

@@ -827,9 +827,10 @@ void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint
     switch (fmt) {
     case F16:  launch_gemm16_fmt<F16, true>(L, A, C, M, out_f32); break;
     case BF16: launch_gemm16_fmt<BF16, false>(L, A, C, M, out_f32); break;
-    case I8:   launch_gemm16_fmt<I8, false>(L, A, C, M, out_f32); break;
-    case I4:   launch_gemm16_fmt<I4, false>(L, A, C, M, out_f32); break;
-    default:   launch_gemm16_fmt<I2, false>(L, A, C, M, out_f32); break;    // FP32 weights never come here
+    // integer codes are exact in either 16-bit type; FP16 keeps 11 bits of the activations instead of 8
+    case I8:   launch_gemm16_fmt<I8, true>(L, A, C, M, out_f32); break;
+    case I4:   launch_gemm16_fmt<I4, true>(L, A, C, M, out_f32); break;
+    default:   launch_gemm16_fmt<I2, true>(L, A, C, M, out_f32); break;     // FP32 weights never come here
     }
 }
 
@@ -888,7 +889,7 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
 {
     const bool keep = (flags & SPHIP_KEEP_LAYERS) != 0;
     const Regime reg = pick_regime(net, n, flags);
-    const bool f16t = net->prec == F16;
+    const bool f16t = net->prec != BF16;          // 16-bit activation type of the matrix-core path
     const uint32_t last = net->layers - 1;
 
     const void *in = d_x;

@@ -33,3 +33,16 @@ def rel_max_abs(got, ref):
     got = np.asarray(got, dtype=np.float64)
     den = np.max(np.abs(ref))
     return float(np.max(np.abs(got - ref)) / (den if den > 0 else 1.0))
+
+
+def argmax_agreement(got, want):
+    """(raw, decided): raw = fraction of rows with the same argmax; decided = the
+    same fraction over rows whose reference top-2 gap exceeds twice the largest
+    absolute deviation of this run.  A flip outside that band cannot be rounding."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    same = got.argmax(1) == want.argmax(1)
+    err = np.max(np.abs(got - want))
+    top2 = np.sort(want, axis=1)[:, -2:]
+    decided = (top2[:, 1] - top2[:, 0]) > 2.0 * err
+    return float(same.mean()), float(same[decided].mean()) if decided.any() else 1.0

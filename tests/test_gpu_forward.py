@@ -1,0 +1,277 @@
+"""Forward parity of the HIP path against the CPU oracle, through the C-ABI.
+
+Tolerances (relative max-abs = max|gpu - ref| / max|ref|):
+  vector path (n <= 64) and FP32 weights ........ 1e-4
+  16-bit matrix-core path (n > 64) .............. 2e-2
+
+Argmax agreement on the matrix-core path: the nets here are random, so many
+samples have two nearly equal top outputs and a rounding-sized perturbation
+flips them.  Two figures are checked: `decided` (rows whose reference top-2 gap
+exceeds twice the largest deviation of the run) must agree 100 %; `raw` (all
+rows) must reach 99.9 % for the integer formats, whose matrix-core path keeps
+FP16 activations, and 98.5 % for BF16 weights (8-bit activations; measured
+99.0-99.7 % on random 10- and 1000-class nets).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from helpers import ALL_ACTS, FORMATS, argmax_agreement, make_oracle_net, quantized_pair, rel_max_abs
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+E = np.load(os.path.join(GOLD, "expected.npz"))
+F32 = np.float32
+TOL_VEC, TOL_MFMA = 1e-4, 2e-2
+
+
+def sphip_forward(S, net, X, flags):
+    """sphip_forward on the net's device handle (to pick the path regardless of n)."""
+    h = S.lib().spingalett_hip_handle(net)
+    assert h, S.last_error()
+    nc = net.contents
+    X = np.ascontiguousarray(X, dtype=F32)
+    out = np.empty((X.shape[0], nc.topology[nc.layers - 1]), dtype=F32)
+    rc = S.lib().sphip_forward(h, X.ctypes.data, X.shape[0], out.ctypes.data, flags)
+    assert rc == 0, S.lib().sphip_last_error_string()
+    return out
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_golden_nets(S, fmt):
+    net = S.load_spingalett(os.path.join(GOLD, f"tiny_{fmt}.nn"))
+    X, want = E["tiny_X"], E[f"tiny_{fmt}_Y"]
+    for i in range(X.shape[0]):                                   # public forward(), one sample
+        y = S.forward(net, X[i])
+        assert y is not None, S.last_error()
+        assert rel_max_abs(y, want[i]) <= TOL_VEC
+    assert rel_max_abs(S.forward_batch(net, X), want) <= TOL_VEC  # batched entry, vector path
+    got = sphip_forward(S, net, X, S.SPHIP_FORCE_GEMM)            # matrix-core path on the same inputs
+    assert rel_max_abs(got, want) <= (TOL_VEC if fmt == "f32" else TOL_MFMA)
+    S.free_network(net)
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "i4"])
+def test_golden_softmax_net(S, fmt):
+    net = S.load_spingalett(os.path.join(GOLD, f"soft_{fmt}.nn"))
+    X, want = E["soft_X"], E[f"soft_{fmt}_Y"]
+    assert rel_max_abs(S.forward_batch(net, X), want) <= TOL_VEC
+    got = sphip_forward(S, net, X, S.SPHIP_FORCE_GEMM)
+    assert rel_max_abs(got, want) <= TOL_MFMA
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+    S.free_network(net)
+
+
+def test_forward_leaves_every_layer_in_neurons(S, O):
+    """forward() mirrors all activations into net->neurons and returns a pointer
+    into it (Network.c:214-250)."""
+    with open(os.path.join(GOLD, "tiny_i8.nn"), "rb") as f:
+        ref = O.Net.parse(f.read())
+    net = S.load_spingalett(os.path.join(GOLD, "tiny_i8.nn"))
+    x = E["tiny_X"][2]
+    y = S.forward(net, x)
+    nc = net.contents
+    neurons = S.neurons_view(net)
+    assert y.ctypes.data == C.addressof(nc.neurons.contents) + 4 * nc.neuron_offsets[3]
+    assert np.array_equal(neurons[:37], x)
+    # layer by layer against the oracle
+    a = x.astype(np.float64)
+    off = 37
+    for l, act in enumerate(ref.act):
+        pre = ref.W(l).astype(np.float64) @ a + ref.b(l)
+        a = O.activate(pre.astype(F32), act).astype(np.float64)
+        w = ref.topology[l + 1]
+        assert rel_max_abs(neurons[off:off + w], a) <= TOL_VEC
+        off += w
+    S.free_network(net)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("act", ALL_ACTS)
+def test_every_activation_every_format(S, O, fmt, act):
+    # hidden layer carries the activation under test (softmax included), aligned and odd widths
+    for topo in ([64, 96, 32], [45, 77, 13]):
+        src = make_oracle_net(O, topo, [act, "none"], seed=11)
+        _, ref, net = quantized_pair(O, S, src, fmt)
+        rng = np.random.default_rng(12)
+        X = (rng.standard_normal((9, topo[0])) * 1.5).astype(F32)
+        want = ref.forward_batch_f64(X)
+        assert rel_max_abs(S.forward_batch(net, X), want) <= TOL_VEC, (topo, "gemv")
+        got = sphip_forward(S, net, X, S.SPHIP_FORCE_GEMM)
+        assert rel_max_abs(got, want) <= (TOL_VEC if fmt == "f32" else TOL_MFMA), (topo, "gemm")
+        S.free_network(net)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 7, 8, 9, 33, 64])
+def test_vector_path_batch_sizes(S, O, n):
+    src = make_oracle_net(O, [256, 512, 128, 10], ["relu", "tanh", "softmax"], seed=2)
+    _, ref, net = quantized_pair(O, S, src, "i4")
+    X = np.random.default_rng(n).standard_normal((n, 256)).astype(F32)
+    got = S.forward_batch(net, X)
+    assert rel_max_abs(got, ref.forward_batch_f64(X)) <= TOL_VEC
+    # every row equals the single-sample forward of that row
+    y0 = S.forward(net, X[n // 2]).copy()
+    assert rel_max_abs(got[n // 2], y0) <= 2e-6
+    S.free_network(net)
+
+
+@pytest.mark.parametrize("fmt", ["f16", "bf16", "i8", "i4", "i2"])
+def test_crossover_agreement(S, O, fmt):
+    """n = 64 runs the vector path, n = 65 the matrix-core path: same net, same rows."""
+    src = make_oracle_net(O, [128, 256, 192, 16], ["leaky_relu", "foo52", "softmax"], seed=4)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    X = np.random.default_rng(5).standard_normal((65, 128)).astype(F32)
+    lo = S.forward_batch(net, X[:64])
+    hi = S.forward_batch(net, X)
+    want = ref.forward_batch_f64(X)
+    assert rel_max_abs(lo, want[:64]) <= TOL_VEC
+    assert rel_max_abs(hi, want) <= TOL_MFMA
+    assert rel_max_abs(hi[:64], lo) <= TOL_MFMA
+    S.free_network(net)
+
+
+@pytest.mark.parametrize("n", [1, 256, 4096])
+def test_config2_int8(S, O, n):
+    """784->512->1000->10, INT8 through the serializer, inputs U[0,1)."""
+    src = make_oracle_net(O, [784, 512, 1000, 10], ["relu", "relu", "softmax"], seed=42, bias_std=0.05)
+    _, ref, net = quantized_pair(O, S, src, "i8")
+    X = np.random.default_rng(7).random((n, 784), dtype=F32)
+    want = ref.forward_batch(X)
+    got = S.forward_batch(net, X)
+    if n <= 64:
+        assert rel_max_abs(got, want) <= TOL_VEC
+    else:
+        assert rel_max_abs(got, want) <= TOL_MFMA
+        raw, decided = argmax_agreement(got, want)
+        assert decided == 1.0 and raw >= (0.999 if n >= 4096 else 0.99), (raw, decided)
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-4)
+    S.free_network(net)
+
+
+def test_config1_fp32_batch256(S, O):
+    """FP32 weights, batch 256: FP32 arithmetic end to end, 1e-4."""
+    src = make_oracle_net(O, [784, 512, 1000, 10], ["relu", "relu", "softmax"], seed=42, bias_std=0.05)
+    net = S.new_spingalett(S.LOSS_CROSS_ENTROPY)
+    S.layer(net, 784)
+    S.layer(net, 512, S.ACT_RELU, S.WEIGHT_INITIALIZATION_NONE)
+    S.layer(net, 1000, S.ACT_RELU, S.WEIGHT_INITIALIZATION_NONE)
+    S.layer(net, 10, S.ACT_SOFTMAX, S.WEIGHT_INITIALIZATION_NONE)
+    for l in range(3):                                   # weights written straight into the public arrays
+        S.weights_view(net, l)[:] = src.W(l)
+        S.biases_view(net, l)[:] = src.b(l)
+    X = np.random.default_rng(8).random((256, 784), dtype=F32)
+    want = src.forward_batch(X)
+    got = S.forward_batch(net, X)
+    assert rel_max_abs(got, want) <= TOL_VEC
+    assert np.array_equal(got.argmax(1), want.argmax(1))
+    assert rel_max_abs(S.forward_batch(net, X[:3]), want[:3]) <= TOL_VEC
+    S.free_network(net)
+
+
+@pytest.mark.parametrize("fmt,topo,acts,n", [
+    ("i4", [1024, 2048, 2048, 512], ["relu", "tanh", "none"], 8),            # config 3 scaled down
+    ("i4", [1024, 2048, 2048, 512], ["relu", "tanh", "none"], 64),
+    ("bf16", [1024, 1024, 1024, 1024, 1000], ["leaky_relu", "foo52", "leaky_relu", "softmax"], 1024),  # config 4 scaled
+    ("i2", [512, 1024, 1024, 1000], ["sigmoid", "relu", "softmax"], 1),       # config 5 scaled
+    ("i2", [512, 1024, 1024, 1000], ["sigmoid", "relu", "softmax"], 2048),
+    ("f16", [512, 768, 300], ["tanh", "none"], 300),
+])
+def test_scaled_configs(S, O, fmt, topo, acts, n):
+    init = "xavier" if fmt == "i4" else "he"
+    src = make_oracle_net(O, topo, acts, seed=21, init=init)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    rng = np.random.default_rng(22)
+    X = (rng.random((n, topo[0]), dtype=F32) * 2 - 1) if fmt == "i2" else rng.standard_normal((n, topo[0])).astype(F32)
+    fn, _, setter = O.find_sgemm()
+    _, want = ref.time_forward_batch(X, 1, fn, 8)        # threaded BLAS leg of the oracle (same call sequence)
+    got = S.forward_batch(net, X)
+    tol = TOL_VEC if n <= 64 else TOL_MFMA
+    assert rel_max_abs(got, want) <= tol
+    if acts[-1] == "softmax" and n > 64:
+        raw, decided = argmax_agreement(got, want)
+        assert decided == 1.0 and raw >= (0.985 if fmt == "bf16" else 0.995), (raw, decided)
+    S.free_network(net)
+
+
+def test_batch_permutation_and_row_independence(S, O):
+    """Samples are independent: permuting the batch permutes the outputs bit for bit."""
+    src = make_oracle_net(O, [256, 384, 64], ["foo52", "softmax"], seed=31)
+    _, ref, net = quantized_pair(O, S, src, "i8")
+    rng = np.random.default_rng(32)
+    X = rng.standard_normal((333, 256)).astype(F32)
+    perm = rng.permutation(333)
+    a = S.forward_batch(net, X)
+    b = S.forward_batch(net, X[perm])
+    assert np.array_equal(a[perm], b)
+    S.free_network(net)
+
+
+def test_device_resident_entry_and_argument_checks(S, O):
+    src = make_oracle_net(O, [128, 64, 8], ["relu", "none"], seed=41)
+    _, ref, net = quantized_pair(O, S, src, "bf16")
+    X = np.random.default_rng(42).standard_normal((100, 128)).astype(F32)
+    d_x = S.DeviceBuffer.from_numpy(X)
+    d_y = S.DeviceBuffer(100 * 8 * 4)
+    assert S.lib().spingalett_forward_batch_device(net, d_x.ptr, 100, d_y.ptr) == 0
+    assert S.lib().spingalett_hip_synchronize() == 0
+    got = d_y.to_numpy(F32, (100, 8))
+    assert np.array_equal(got, S.forward_batch(net, X))
+    assert S.lib().spingalett_forward_batch_device(net, None, 100, d_y.ptr) == 1
+    assert S.last_error()[0] == S.SPINGALETT_ERR_INVALID
+    S.clear_error()
+    assert S.lib().spingalett_forward_batch_device(None, d_x.ptr, 100, d_y.ptr) == 1
+    S.clear_error()
+    assert S.lib().spingalett_forward_batch(net, None, 3, got.ctypes.data) is None
+    assert S.last_error()[0] == 0                                   # silent, like forward()
+    S.free_network(net)
+
+
+def test_zero_scale_arrays_forward_to_bias_only(S, O):
+    """An all-zero weight matrix is written with scale 0 and decodes to zeros
+    (Serialize.c:231-236): the layer outputs act(bias)."""
+    src = make_oracle_net(O, [32, 16], ["none"], seed=51)
+    src.W(0)[:] = 0
+    _, ref, net = quantized_pair(O, S, src, "i4")
+    X = np.random.default_rng(52).standard_normal((3, 32)).astype(F32)
+    got = S.forward_batch(net, X)
+    assert np.allclose(got, np.broadcast_to(ref.b(0), (3, 16)), rtol=1e-6, atol=0)
+    S.free_network(net)
+
+
+def test_full_size_layer_unit_vector_probe(S):
+    """16384 x 16384 INT4 (the largest layer of config 3, 128 MiB of codes):
+    x = e_k reads column k of W exactly, and f(2x) = 2 f(x) for a bias-free
+    linear layer — properties that hold at any size."""
+    K = N = 16384
+    rng = np.random.default_rng(61)
+    codes = rng.integers(0, 256, size=N * K // 2, dtype=np.uint8)
+    mx = 7.0                                                         # scale max/7 = 1: outputs are the integer codes
+    net = S.DeviceNet([K, N], [S.ACT_NONE], S.PRECISION_INT4)
+    net.upload(0, 0, codes, mx)
+    net.upload(0, 1, np.zeros(N // 2, np.uint8), 0.0)
+    ks = [0, 1, 7, 4095, 8192, 16383]
+    X = np.zeros((len(ks), K), F32)
+    for i, k in enumerate(ks):
+        X[i, k] = 1.0
+    got = net.forward(X)
+    rows = codes.reshape(N, K // 2)
+    for i, k in enumerate(ks):
+        nib = (rows[:, k // 2] >> ((k & 1) * 4)) & 15
+        q = nib.astype(np.int32) - np.where(nib & 8, 16, 0)
+        assert np.array_equal(got[i], q.astype(F32)), k
+    x = rng.standard_normal((1, K)).astype(F32)
+    y1, y2 = net.forward(x), net.forward(2 * x)
+    assert np.array_equal(2 * y1, y2)
+    # and the matrix-core path reads the same codes: one-hot rows are exact in bf16
+    Xg = np.zeros((65, K), F32)
+    Xg[np.arange(65), np.arange(65) * 251] = 1.0
+    gg = net.forward(Xg)
+    for i in (0, 17, 64):
+        k = i * 251
+        nib = (rows[:, k // 2] >> ((k & 1) * 4)) & 15
+        q = nib.astype(np.int32) - np.where(nib & 8, 16, 0)
+        assert np.array_equal(gg[i], q.astype(F32)), k
+    net.destroy()

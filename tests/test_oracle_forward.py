@@ -1,0 +1,109 @@
+"""Pins the oracle's forward (GEMV/GEMM + bias + activation) against float64
+brute force, closed forms and invariants — none of which restate its loops."""
+import os
+
+import numpy as np
+import pytest
+from scipy import special
+
+from helpers import ALL_ACTS, make_oracle_net
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+E = np.load(os.path.join(GOLD, "expected.npz"))
+F32 = np.float32
+
+
+def test_piecewise_linear_activations_closed_form(O):
+    x = np.array([-3.0, -1.0, -0.0, 0.0, 0.25, 1.0, 1.5, 10.0], dtype=F32)
+    a = F32(0.01)
+    assert np.array_equal(O.activate(x, O.ACT["relu"]), np.maximum(x, 0))
+    assert np.array_equal(O.activate(x, O.ACT["leaky_relu"]), np.where(x > 0, x, a * x))
+    assert np.array_equal(O.activate(x, O.ACT["foo52"]),
+                          np.where(x > 1, F32(1) + a * (x - F32(1)), np.where(x < 0, a * x, x)).astype(F32))
+    assert np.array_equal(O.activate(x, O.ACT["none"]), x)
+
+
+def test_transcendental_activations_against_library(O):
+    x = np.linspace(-12, 12, 4001).astype(F32)
+    assert np.allclose(O.activate(x, O.ACT["sigmoid"]), special.expit(x.astype(np.float64)), rtol=3e-7, atol=1e-9)
+    assert np.allclose(O.activate(x, O.ACT["tanh"]), np.tanh(x.astype(np.float64)), rtol=3e-7, atol=1e-9)
+    s = O.activate(x, O.ACT["sigmoid"])
+    assert np.allclose(s + s[::-1], 1.0, atol=2e-7)                 # sigmoid(-x) = 1 - sigmoid(x)
+
+
+def test_softmax_invariants(O):
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal((6, 1000)) * 4).astype(F32)
+    y = O.activate(x, O.ACT["softmax"])
+    assert np.allclose(y.sum(axis=1), 1.0, atol=1e-5)
+    assert np.array_equal(y.argmax(axis=1), x.argmax(axis=1))
+    assert np.allclose(y, special.softmax(x.astype(np.float64), axis=1), rtol=2e-5, atol=1e-9)
+    shifted = O.activate(x + F32(3.0), O.ACT["softmax"])
+    assert np.allclose(shifted, y, rtol=1e-4, atol=1e-9)
+    # rows are independent: a huge value in one row must not leak into another
+    x2 = x.copy(); x2[0, 0] = 80.0
+    y2 = O.activate(x2, O.ACT["softmax"])
+    assert np.array_equal(y2[1:], y[1:]) and y2[0, 0] > 0.999999
+
+
+@pytest.mark.parametrize("fmt", ["f32", "f16", "bf16", "i8", "i4", "i2"])
+def test_golden_forward_outputs(O, fmt):
+    with open(os.path.join(GOLD, f"tiny_{fmt}.nn"), "rb") as f:
+        net = O.Net.parse(f.read())
+    X = E["tiny_X"]
+    want = E[f"tiny_{fmt}_Y"]                                  # numpy float64, independent of the oracle
+    assert np.allclose(net.forward_batch(X), want, rtol=2e-6, atol=2e-7)
+    assert np.allclose(net.forward_batch_f64(X), want, rtol=1e-12, atol=1e-14)
+    for i in range(X.shape[0]):
+        assert np.allclose(net.forward_single(X[i]), want[i], rtol=2e-6, atol=2e-7)
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "i4"])
+def test_golden_softmax_net(O, fmt):
+    with open(os.path.join(GOLD, f"soft_{fmt}.nn"), "rb") as f:
+        net = O.Net.parse(f.read())
+    want = E[f"soft_{fmt}_Y"]
+    assert np.allclose(net.forward_batch(E["soft_X"]), want, rtol=5e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("act", ALL_ACTS)
+def test_each_activation_in_a_net_against_numpy(O, act):
+    net = make_oracle_net(O, [19, 33, 11], [act, "none"], seed=5)
+    rng = np.random.default_rng(1)
+    X = rng.standard_normal((7, 19)).astype(F32)
+    h = X.astype(np.float64) @ net.W(0).astype(np.float64).T + net.b(0)
+    f = {"sigmoid": special.expit, "relu": lambda v: np.maximum(v, 0), "tanh": np.tanh,
+         "leaky_relu": lambda v: np.where(v > 0, v, np.float64(F32(0.01)) * v),
+         "foo52": lambda v: np.where(v > 1, 1 + np.float64(F32(0.01)) * (v - 1), np.where(v < 0, np.float64(F32(0.01)) * v, v)),
+         "softmax": lambda v: special.softmax(v, axis=1), "none": lambda v: v}[act]
+    want = f(h) @ net.W(1).astype(np.float64).T + net.b(1)
+    assert np.allclose(net.forward_batch(X), want, rtol=1e-5, atol=1e-6)
+
+
+def test_layout_is_row_major_out_by_in(O):
+    # a transposed-operand mistake fails: W[j][k] multiplies x[k] and lands in y[j]
+    net = O.Net.new([3, 2], [O.ACT["none"]])
+    net.W(0)[:] = np.array([[1, 2, 3], [10, 20, 30]], dtype=F32)
+    net.b(0)[:] = np.array([0.5, -0.5], dtype=F32)
+    y = net.forward_single(np.array([1, 0, -1], dtype=F32))
+    assert np.array_equal(y, np.array([1 - 3 + 0.5, 10 - 30 - 0.5], dtype=F32))
+    assert np.array_equal(net.weights[:6], np.array([1, 2, 3, 10, 20, 30], dtype=F32))
+
+
+def test_mid_size_against_numpy_matmul(O):
+    net = make_oracle_net(O, [784, 512, 1000, 10], ["relu", "relu", "softmax"], seed=2)
+    rng = np.random.default_rng(3)
+    X = rng.random((16, 784), dtype=F32)
+    a = X.astype(np.float64)
+    for l, act in enumerate(["relu", "relu", "softmax"]):
+        a = a @ net.W(l).astype(np.float64).T + net.b(l)
+        a = special.softmax(a, axis=1) if act == "softmax" else np.maximum(a, 0)
+    got = net.forward_batch(X)
+    assert np.max(np.abs(got - a)) / np.max(np.abs(a)) < 1e-5
+    assert np.array_equal(got.argmax(1), a.argmax(1))
+    sec, out = net.time_forward_batch(X, 1, None, 2)            # built-in threaded GEMM leg
+    assert np.max(np.abs(out - a)) / np.max(np.abs(a)) < 1e-5 and sec > 0
+    fn, desc, setter = O.find_sgemm()
+    if fn is not None:                                          # BLAS leg, when a BLAS is present
+        sec, out = net.time_forward_batch(X, 1, fn, 2)
+        assert np.max(np.abs(out - a)) / np.max(np.abs(a)) < 1e-5
