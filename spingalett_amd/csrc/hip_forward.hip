@@ -15,8 +15,10 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "spingalett_hip.h"
@@ -73,6 +75,11 @@ int fail_hip(const char *what, hipError_t e)
     } while (0)
 
 hipStream_t g_stream = nullptr;
+int g_dbg = 0;
+int g_gemv_variant = 1;     // 0: vector-ALU GEMV only (tuning switch)
+int g_gemv_waves = 0;       // 0: automatic
+int g_gemv_lds_kib = 64;
+int g_gemm_variant = 1;     // 0: 128x128 tiles only; 1: 256x256 / 8 waves; 2: 256x256 / 4 waves (tuning switch)
 
 int ensure_stream()
 {
@@ -82,6 +89,11 @@ int ensure_stream()
     if (cnt <= 0) return fail_msg("no HIP device");
     HCHECK(hipSetDevice(0));
     HCHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    if (const char *v = getenv("SPHIP_GEMM_VARIANT")) g_gemm_variant = atoi(v);
+    if (const char *v = getenv("SPHIP_DBG")) g_dbg = atoi(v);
+    if (const char *v = getenv("SPHIP_GEMV_VARIANT")) g_gemv_variant = atoi(v);
+    if (const char *v = getenv("SPHIP_GEMV_WAVES")) g_gemv_waves = atoi(v);
+    if (const char *v = getenv("SPHIP_GEMV_LDS")) g_gemv_lds_kib = atoi(v);
     return 0;
 }
 
@@ -195,6 +207,13 @@ __device__ __forceinline__ uint16_t f32_to_t16(float x)
 }
 
 __device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum_i(int v)
 {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
@@ -403,6 +422,306 @@ __global__ __launch_bounds__(256) void sp_gemv_generic(const LayerArgs L, const 
 }
 
 // ---------------------------------------------------------------------------
+// Integer-weight GEMV on the INT8 matrix cores (n <= 64, INT8 / INT4 / INT2)
+// ---------------------------------------------------------------------------
+// The packed codes are (nearly) MFMA operands already: INT8 bytes as they are,
+// INT4 / INT2 after a mask-and-shift that leaves one code per byte.  The FP32
+// activations are turned into exact integers instead of the weights into floats:
+// per sample and K chunk, X = rint(x * 2^p) with |X| < 2^22, written as three
+// balanced base-256 digits d0 + 256 d1 + 65536 d2, each an INT8.  Then
+//     sum_k q_k x_k = 2^-p * (S0 + 256 S1 + 65536 S2),  S_i = sum_k q_k d_i,k
+// and the S_i are exact INT32 dot products from v_mfma_i32_16x16x64_i8.  One
+// 16-row A tile carries four samples (three digit rows + one zero row each), the
+// B operand is 16 weight rows x 64 codes, so a wave needs no reduction across
+// lanes: lane (n, s) ends up holding S0, S1, S2 of output row n and sample s.
+// The unsigned fields of INT4 / INT2 are biased codes (q + 8, q + 2 after an XOR
+// of the sign bits); the bias is removed exactly with sum_k d_i,k.
+//
+// Work split: a wave owns 16 output rows over the whole K; the waves of a
+// workgroup (1, 2 or 4, chosen so that the grid fills the chip) share the digit
+// planes of the current K chunk in LDS.  No workgroup ever waits for another:
+// device-scope fences cost an L2 write-back on this multi-die part.
+struct GemvI8Args {
+    LayerArgs L;
+    const float *x;        // [nb][K] activations (quantise kernel)
+    uint8_t *aq;           // digit planes, see sp_quant_x
+    float *inv;            // [chunks][nb] 2^-p
+    int *dsum;             // [chunks][nb][4] digit sums (bias removal)
+    float *y;              // [nb][N]
+    int nb;
+    uint32_t kc;           // K chunk = one scale block (multiple of the 64-byte block)
+    uint32_t nchunks;      // ceil(K / kc)
+    uint32_t stage_blocks; // 64-byte blocks whose digit planes are held in LDS at a time
+    uint32_t rw, ks;       // waves of a workgroup: row groups x K shares
+    uint32_t meta_bytes;   // LDS bytes of the per-chunk scale records (multiple of 16)
+};
+
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+
+template <int FMT>
+struct I8Fmt {
+    static constexpr int bits = fmt_bits(FMT);
+    static constexpr int KL = 512 / bits;      // codes per 64-byte row segment (one wave load)
+    static constexpr int NMF = KL / 64;        // MFMAs one lane-load feeds
+    static constexpr int WK = 32 / bits;       // codes per 32-bit word
+    static constexpr int BIAS = FMT == I8 ? 0 : FMT == I4 ? 8 : 2;
+};
+
+// Quantise kernel: grid (chunks, nb), one workgroup per sample and scale chunk.
+// Output order = the order the A operand is read.  A 64-byte weight segment
+// (block) is spread over 4 lane groups g of 16 bytes = 4 words w; word w holds
+// WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
+//   INT8: 4w+i (u = 0)      INT4: 8w + 2i + u      INT2: 16w + 4i + u
+// of the lane group.  Per (block, u, g) the planes are stored as
+//   [sample][digit 0..2][16 bytes]
+// i.e. 3 bytes per element and sample; the GEMV kernel copies them verbatim.
+template <int FMT>
+__global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK;
+    __shared__ float s_red[4];
+    __shared__ int s_sum[3];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t ch = blockIdx.x, s0 = blockIdx.y, K = a.L.K;
+    const uint32_t k0 = ch * a.kc;
+    const uint32_t klen = k0 + a.kc <= K ? a.kc : K - k0;
+    const uint32_t nblk = a.kc / KL;                         // blocks per chunk (last chunk zero-padded)
+    const float *xs = a.x + (size_t)s0 * K + k0;
+
+    float m = 0.0f;
+    for (uint32_t k = t; k < klen; k += 256) m = fmaxf(m, fabsf(xs[k]));
+    m = wave_max(m);
+    if (lane == 0) s_red[wave] = m;
+    if (t < 3) s_sum[t] = 0;
+    __syncthreads();
+    const float amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
+    if (e < -126) e = -126;
+    int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
+    p = p > 126 ? 126 : p;
+    const bool live = amax > 0.0f && amax < 3.0e38f;         // zero, inf and NaN chunks contribute nothing
+    const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
+
+    int ds0 = 0, ds1 = 0, ds2 = 0;
+    const uint32_t nwords = nblk * (KL / WK);                // weight words per chunk row
+    for (uint32_t wi = t; wi < nwords; wi += 256) {
+        const uint32_t blk = wi / (KL / WK), r = wi % (KL / WK), g = r >> 2, w = r & 3u;
+        const uint32_t kw = blk * KL + g * (KL / 4) + w * WK;      // first code of this word
+        uint32_t d0w[NMF], d1w[NMF], d2w[NMF];
+#pragma unroll
+        for (int u = 0; u < NMF; ++u) d0w[u] = d1w[u] = d2w[u] = 0;
+#pragma unroll
+        for (int c = 0; c < WK; ++c) {
+            const uint32_t k = kw + c;
+            int X = 0;
+            if (k < klen) X = (int)rintf(xs[k] * scale);
+            const int d0 = (int)(int8_t)(X & 255);
+            const int X1 = (X - d0) >> 8;
+            const int d1 = (int)(int8_t)(X1 & 255);
+            const int d2 = (X1 - d1) >> 8;
+            ds0 += d0; ds1 += d1; ds2 += d2;
+            const int u = c % NMF, i = c / NMF;              // code c of the word -> MFMA u, byte i
+            d0w[u] |= (uint32_t)(d0 & 255) << (8 * i);
+            d1w[u] |= (uint32_t)(d1 & 255) << (8 * i);
+            d2w[u] |= (uint32_t)(d2 & 255) << (8 * i);
+        }
+#pragma unroll
+        for (int u = 0; u < NMF; ++u) {
+            uint8_t *dst = a.aq + (((((size_t)ch * nblk + blk) * NMF + u) * 4 + g) * (size_t)a.nb + s0) * 48 + w * 4;
+            *reinterpret_cast<uint32_t *>(dst) = d0w[u];
+            *reinterpret_cast<uint32_t *>(dst + 16) = d1w[u];
+            *reinterpret_cast<uint32_t *>(dst + 32) = d2w[u];
+        }
+    }
+    ds0 = wave_sum_i(ds0);
+    ds1 = wave_sum_i(ds1);
+    ds2 = wave_sum_i(ds2);
+    if (lane == 0) {
+        atomicAdd(&s_sum[0], ds0);
+        atomicAdd(&s_sum[1], ds1);
+        atomicAdd(&s_sum[2], ds2);
+    }
+    __syncthreads();
+    if (t == 0) {
+        a.inv[(size_t)ch * a.nb + s0] = live ? __uint_as_float((uint32_t)(127 - p) << 23) : 0.0f;
+        int *d = a.dsum + ((size_t)ch * a.nb + s0) * 4;
+        d[0] = s_sum[0]; d[1] = s_sum[1]; d[2] = s_sum[2]; d[3] = 0;
+    }
+}
+
+// MT = 16-row A tiles (four samples each).  Rows of D that belong to no sample
+// (fourth row of a slot, slots beyond nb) are never read, so their lanes may load
+// anything: they are pointed at the start of the block.
+// The waves of a workgroup are rw row groups x ks K shares (wave = ks_id * rw +
+// rw_id); share ks_id takes the 64-byte blocks ks_id, ks_id + ks, ... of its rows.
+// Weights are fetched in groups of four blocks, the next group in flight while
+// the current one is multiplied; scale chunks are whole numbers of groups.
+template <int FMT, int MT>
+__global__ __launch_bounds__(MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, G = 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    // [nchunks][nb] {2^-p bits, d0 sum, d1 sum, d2 sum}, then the digit planes of one stage:
+    // [stage blocks][NMF][4 g][nb][3][16 bytes]
+    int4 *meta = reinterpret_cast<int4 *>(lds_all);
+    uint8_t *A_lds = lds_all + a.meta_bytes;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t N = a.L.N, K = a.L.K;
+    const int nb = a.nb;
+    const uint32_t rw = a.rw, ks = a.ks, ks_id = (uint32_t)wave / rw, rw_id = (uint32_t)wave % rw;
+    const uint32_t nrow = (blockIdx.x * rw + rw_id) * 16u + (lane & 15);
+    const uint32_t g = lane >> 4;
+    const size_t row_bytes = (size_t)K * F::bits / 8u;
+    const uint8_t *wrow = a.L.w + (size_t)(nrow < N ? nrow : N - 1) * row_bytes + g * 16u + ks_id * 64u;
+    // largest offset (from wrow) whose 16 bytes stay inside the row; reads past it are clamped there
+    // and meet zero digits
+    const int64_t row_last = (int64_t)row_bytes - 16 - (int64_t)(g * 16u + ks_id * 64u);
+    const uint32_t kcb = a.kc / KL;                           // blocks per scale chunk
+    const uint32_t blk_bytes = (uint32_t)NMF * 4u * (uint32_t)nb * 48u;   // digit planes of one block
+    const uint32_t u_bytes = 4u * (uint32_t)nb * 48u;
+    const uint32_t qstep = ks * 64u;                          // byte distance of this wave's consecutive blocks
+    const uint32_t groups_per_chunk = kcb / (ks * G);         // host guarantees divisibility
+    const uint32_t chunks_per_stage = a.stage_blocks / kcb;
+
+    uint32_t a_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t m = lane & 15u, slot = (uint32_t)mt * 4u + (m >> 2), d = m & 3u;
+        a_off[mt] = (slot < (uint32_t)nb && d < 3u) ? ((g * (uint32_t)nb + slot) * 3u + d) * 16u : 0u;
+    }
+
+    float yacc[MT];
+    i32x4v acc[2][MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        yacc[mt] = 0.0f;
+        acc[0][mt] = acc[1][mt] = (i32x4v){0, 0, 0, 0};
+    }
+
+    auto load_blk = [&](uint32_t q) {                          // q-th block of this wave
+        int64_t off = (int64_t)q * qstep;
+        off = off < row_last ? off : row_last;
+        off = off > 0 ? off : 0;
+        return *reinterpret_cast<const uint4 *>(wrow + off);
+    };
+    auto process = [&](const uint4 wv, const uint8_t *rec) {
+        const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+        i32x4v bop[NMF];
+        if constexpr (FMT == I8) {
+            bop[0] = (i32x4v){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        } else if constexpr (FMT == I4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x8 = w[q] ^ 0x88888888u;          // nibble -> q + 8
+                bop[0][q] = (int)(x8 & 0x0F0F0F0Fu);
+                bop[1][q] = (int)((x8 >> 4) & 0x0F0F0F0Fu);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x2 = w[q] ^ 0xAAAAAAAAu;          // field -> q + 2
+                bop[0][q] = (int)(x2 & 0x03030303u);
+                bop[1][q] = (int)((x2 >> 2) & 0x03030303u);
+                bop[2][q] = (int)((x2 >> 4) & 0x03030303u);
+                bop[3][q] = (int)((x2 >> 6) & 0x03030303u);
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < NMF; ++f)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const i32x4v aop = *reinterpret_cast<const i32x4v *>(rec + f * u_bytes + a_off[mt]);
+                acc[f & 1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, bop[f], acc[f & 1][mt], 0, 0, 0);
+            }
+    };
+    auto fold = [&](uint32_t ch) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int s0 = mt * 4 + (int)g;
+            if (s0 < nb) {
+                const int4 md = meta[(size_t)ch * nb + s0];
+                int S0 = acc[0][mt][0] + acc[1][mt][0], S1 = acc[0][mt][1] + acc[1][mt][1], S2 = acc[0][mt][2] + acc[1][mt][2];
+                if (F::BIAS != 0 && ks_id == 0) {       // one K share removes the code bias of the whole chunk
+                    S0 -= F::BIAS * md.y;
+                    S1 -= F::BIAS * md.z;
+                    S2 -= F::BIAS * md.w;
+                }
+                const float tsum = fmaf((float)S2, 65536.0f, fmaf((float)S1, 256.0f, (float)S0));
+                yacc[mt] = fmaf(tsum, __int_as_float(md.x), yacc[mt]);
+            }
+            acc[0][mt] = acc[1][mt] = (i32x4v){0, 0, 0, 0};
+        }
+    };
+
+    // first weight group goes out before anything else
+    uint4 nxt[G];
+#pragma unroll
+    for (int u = 0; u < G; ++u) nxt[u] = load_blk((uint32_t)u);
+
+    // scale records of all chunks
+    for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
+        const int *d = a.dsum + (size_t)i * 4;
+        meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
+    }
+
+    uint32_t q = 0;                                            // this wave's block counter
+    for (uint32_t ch0 = 0; ch0 < a.nchunks; ch0 += chunks_per_stage) {
+        const uint32_t nch = ch0 + chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks - ch0;
+        if (ch0) __syncthreads();                             // previous stage fully consumed
+        {
+            const uint4 *src = reinterpret_cast<const uint4 *>(a.aq + (size_t)ch0 * kcb * blk_bytes);
+            const uint32_t pieces = nch * kcb * (blk_bytes / 16u);
+            for (uint32_t i = t; i < pieces; i += nthreads) reinterpret_cast<uint4 *>(A_lds)[i] = src[i];
+        }
+        __syncthreads();
+        const uint8_t *rec = A_lds + (size_t)ks_id * blk_bytes;
+        const size_t rstep = (size_t)ks * blk_bytes;
+        for (uint32_t ch = ch0; ch < ch0 + nch; ++ch) {
+            for (uint32_t gi = 0; gi < groups_per_chunk; ++gi) {
+                uint4 cur[G];
+#pragma unroll
+                for (int u = 0; u < G; ++u) cur[u] = nxt[u];
+                q += G;
+#pragma unroll
+                for (int u = 0; u < G; ++u) nxt[u] = load_blk(q + u);
+#pragma unroll
+                for (int u = 0; u < G; ++u) process(cur[u], rec + (size_t)u * rstep);
+                rec += G * rstep;
+            }
+            fold(ch);
+        }
+    }
+
+    // add the K shares of a row group (in share order) through LDS
+    if (ks > 1) {
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(A_lds);         // [ks][rw][MT][64]
+        if (ks_id > 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) red[(((size_t)ks_id * rw + rw_id) * MT + mt) * 64 + lane] = yacc[mt];
+        }
+        __syncthreads();
+        if (ks_id > 0) return;
+        for (uint32_t o = 1; o < ks; ++o)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) yacc[mt] += red[(((size_t)o * rw + rw_id) * MT + mt) * 64 + lane];
+    }
+
+    if (nrow < N) {
+        const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, nrow) * a.L.bscale;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int s0 = mt * 4 + (int)g;
+            if (s0 < nb) a.y[(size_t)s0 * N + nrow] = apply_act(fmaf(yacc[mt], a.L.wscale, bias), a.L.act);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // softmax over rows (Activation.c:5-21); one wave per row
 // ---------------------------------------------------------------------------
 // out_kind: 0 FP32, 1 BF16, 2 FP16
@@ -458,6 +777,7 @@ struct GemmArgs {
     void *C;               // [M][N] 16-bit, or FP32 when out_f32
     uint32_t M;
     int out_f32;
+    int dbg;
 };
 
 // (float)q as a 16-bit float; exact for |q| <= 128 in either type
@@ -661,6 +981,445 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     }
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int OFF>
+__device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
+
+// CNT fragments 2 KiB apart (32 tile rows of 64 bytes) starting at addr + BASE
+template <int BASE, int CNT, int I = 0>
+__device__ __forceinline__ void frag_reads64(u32x4 *dst, uint32_t addr)
+{
+    if constexpr (I < CNT) {
+        ds_read128<BASE + I * 2048>(dst[I], addr);
+        frag_reads64<BASE, CNT, I + 1>(dst, addr);
+    }
+}
+
+template <int OFF>
+__device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+
+// reads CNT fragments 4 KiB apart (32 tile rows of 128 bytes) starting at addr + BASE
+template <int BASE, int CNT, int I = 0>
+__device__ __forceinline__ void frag_reads(u32x4 *dst, uint32_t addr)
+{
+    if constexpr (I < CNT) {
+        ds_read128<BASE + I * 4096>(dst[I], addr);
+        frag_reads<BASE, CNT, I + 1>(dst, addr);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Large-tile variant of the 16-bit MFMA GEMM (K a multiple of 64, rows 16-byte
+// aligned).  WM x WN waves, each TM x TN tiles of 32x32; BK = 64.
+//   * LDS rows hold 64 elements = eight 16-byte chunks, unpadded; chunk c of row
+//     r sits at position c ^ ((r >> 1) & 7).  A 128-bit fragment read is served 16
+//     lanes (16 consecutive rows, 256 bytes = all 64 banks) per cycle: rows of equal
+//     parity share a 128-byte half, and r >> 1 gives those eight rows eight
+//     different chunk positions.
+//   * 16-bit operands (activations always, BF16/FP16 weights) go from global
+//     memory straight into LDS (global_load_lds_dwordx4: each wave fills 1 KiB =
+//     8 tile rows per instruction); which global chunk a lane fetches carries the
+//     swizzle.  Integer weights pass through registers to be unpacked.
+//   * two LDS stages: tile kt+1 is in flight while tile kt feeds the MFMAs; one
+//     barrier per K tile.
+template <int FMT, bool F16T, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
+{
+    constexpr int NT = 64 * WM * WN, NWAVES = WM * WN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 64;
+    constexpr int bits = fmt_bits(FMT);
+    constexpr bool W_DIRECT = (FMT == BF16 || FMT == F16);
+    constexpr int A_ISSUES = BM * 8 / NT;               // 16-byte chunks per thread and tile
+    constexpr int W_ISSUES = BN * 8 / NT;
+    constexpr int EPL = 128 / bits;                     // weight elements per 16-byte global load
+    constexpr int CPL = EPL / 8;                        // LDS chunks produced per global load
+    constexpr int W_LOADS = W_DIRECT ? 1 : (BN * BK / EPL + NT - 1) / NT;
+
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    uint16_t *As = smem;                                // [2][BM][64]
+    uint16_t *Ws = smem + 2 * BM * BK;                  // [2][BN][64]
+
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // tile order: each XCD (workgroup id mod 8) gets a contiguous run of tiles; inside
+    // the run, 8 row tiles x 4 column tiles are consecutive so that the 32 workgroups
+    // an XCD runs at once share A rows and W rows in its L2
+    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = ntiles / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    uint32_t tm, tn;
+    {
+        constexpr uint32_t GM = 8;
+        const uint32_t group = bid / (GM * tiles_n);
+        const uint32_t first = group * GM;
+        const uint32_t rows = tiles_m - first < GM ? tiles_m - first : GM;
+        const uint32_t in = bid - group * GM * tiles_n;
+        tm = first + in % rows;
+        tn = in / rows;
+    }
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // per-thread global source of each direct-to-LDS issue (k offset added per tile)
+    const uint16_t *a_src[A_ISSUES];
+#pragma unroll
+    for (int i = 0; i < A_ISSUES; ++i) {
+        const int ci = (i * NWAVES + wave) * 64 + lane, row = ci >> 3, pos = ci & 7;
+        const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+        a_src[i] = g.A + (size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3);
+    }
+    const uint16_t *w_src[W_DIRECT ? W_ISSUES : 1];
+    if constexpr (W_DIRECT) {
+#pragma unroll
+        for (int i = 0; i < W_ISSUES; ++i) {
+            const int ci = (i * NWAVES + wave) * 64 + lane, row = ci >> 3, pos = ci & 7;
+            const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+            w_src[i] = reinterpret_cast<const uint16_t *>(g.L.w) + (size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3);
+        }
+    }
+    const size_t w_row_bytes = (size_t)K * bits / 8u;
+    uint4 rw[W_LOADS];
+
+    auto issue_direct = [&](int buf, uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < A_ISSUES; ++i) {
+            uint16_t *dst = As + buf * BM * BK + (i * NWAVES + wave) * 512;      // 64 chunks x 8 elements
+            __builtin_amdgcn_global_load_lds((const void *)(a_src[i] + k0),
+                                             (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+        }
+        if constexpr (W_DIRECT) {
+#pragma unroll
+            for (int i = 0; i < W_ISSUES; ++i) {
+                uint16_t *dst = Ws + buf * BN * BK + (i * NWAVES + wave) * 512;
+                __builtin_amdgcn_global_load_lds((const void *)(w_src[i] + k0),
+                                                 (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+            }
+        }
+    };
+    auto load_w_regs = [&](uint32_t k0) {
+        if constexpr (!W_DIRECT) {
+            constexpr int LPR = BK / EPL;
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + NT * i, row = c / LPR, kc = c % LPR;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                if (row < BN)
+                    rw[i] = *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)(k0 + kc * EPL) * bits / 8u);
+            }
+        }
+    };
+    auto store_w_regs = [&](int buf) {
+        if constexpr (!W_DIRECT) {
+            constexpr int LPR = BK / EPL;
+            constexpr int PW = 16 / bits;
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + NT * i, row = c / LPR, kc = c % LPR;
+                if (row >= BN) continue;
+                const uint32_t w[4] = {rw[i].x, rw[i].y, rw[i].z, rw[i].w};
+                uint32_t o[4 * PW];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) unpack_word16<FMT, F16T>(w[q], o + q * PW);
+                uint16_t *rowp = Ws + buf * BN * BK + row * BK;
+#pragma unroll
+                for (int v = 0; v < CPL; ++v) {
+                    const int chunk = kc * CPL + v;
+                    *reinterpret_cast<uint4 *>(rowp + ((chunk ^ ((row >> 1) & 7)) << 3)) =
+                        make_uint4(o[4 * v], o[4 * v + 1], o[4 * v + 2], o[4 * v + 3]);
+                }
+            }
+        }
+    };
+
+    // ---- main loop -----------------------------------------------------------
+    // Fragment reads are issued as explicit ds_read_b128 with manual lgkmcnt waits:
+    // the compiler would otherwise drain every pending LDS-DMA load before the first
+    // LDS read of an iteration and serialise load and compute.  Reads of k-step s+1
+    // are in flight while the MFMAs of k-step s run.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)smem;
+    const int h = lane >> 5, l7 = (lane >> 1) & 7;
+    uint32_t va[4], vw[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const uint32_t xo = (uint32_t)(((2 * ks + h) ^ l7) << 4);
+        va[ks] = lds0 + (uint32_t)((wm * TM * 32 + (lane & 31)) * 128) + xo;
+        vw[ks] = lds0 + (uint32_t)(2 * BM * BK * 2) + (uint32_t)((wn * TN * 32 + (lane & 31)) * 128) + xo;
+    }
+    u32x4 fa[2][TM], fb[2][TN];
+
+    auto stage = [&](auto cur_c, bool more, uint32_t knext) {
+        constexpr int CUR = decltype(cur_c)::value;
+        if (more && !(g.dbg & 1)) {
+            issue_direct(CUR ^ 1, knext);
+            load_w_regs(knext);
+        }
+        frag_reads<CUR * BM * BK * 2, TM>(fa[0], va[0]);
+        frag_reads<CUR * BN * BK * 2, TN>(fb[0], vw[0]);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int cs = ks & 1;
+            if (ks < 3) {
+                frag_reads<CUR * BM * BK * 2, TM>(fa[cs ^ 1], va[ks + 1]);
+                frag_reads<CUR * BN * BK * 2, TN>(fb[cs ^ 1], vw[ks + 1]);
+                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+            } else {
+                asm volatile("s_waitcnt lgkmcnt(0)");
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[cs][i]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[cs][j]));
+            __builtin_amdgcn_sched_barrier(0);          // keep the MFMA group between its wait and the next reads
+            if (!(g.dbg & 2))
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (F16T) {
+                        f16x8 a, b;
+                        __builtin_memcpy(&a, &fa[cs][i], 16);
+                        __builtin_memcpy(&b, &fb[cs][j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
+                    } else {
+                        bf16x8 a, b;
+                        __builtin_memcpy(&a, &fa[cs][i], 16);
+                        __builtin_memcpy(&b, &fb[cs][j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
+                    }
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (more) store_w_regs(CUR ^ 1);
+        __syncthreads();       // next stage has landed (the fence drains the LDS DMA), this one is free again
+    };
+
+    const uint32_t ktiles = K / BK;
+    issue_direct(0, 0);
+    load_w_regs(0);
+    store_w_regs(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < ktiles; kt += 2) {
+        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, (kt + 1) * BK);
+        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, (kt + 2) * BK);
+    }
+
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= M) continue;
+                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
+                const size_t o = (size_t)row * N + col;
+                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Streaming variant for 16-bit weights (BF16 / FP16): 256 x 256 tile, BK = 32,
+// four LDS stages, LDS-DMA three tiles ahead.  The memory pipe is never drained:
+// in the middle of stage t each wave waits only until its share of tile t+1 has
+// landed (s_waitcnt vmcnt leaves the younger tile in flight), meets the other
+// waves at one barrier, then queues tile t+3 into the buffer tile t-1 just left
+// and already requests the first fragments of tile t+1.
+// LDS rows hold 32 elements = four 16-byte chunks; chunk c of row r sits at
+// position c ^ ((r >> 2) & 3): the 16 consecutive rows one fragment-read cycle
+// touches (256 bytes = 4 rows of 64 bytes) fall on 16 different 16-byte slots.
+template <bool F16T>
+__global__ __launch_bounds__(512) void sp_gemm16_pipe(const GemmArgs g)
+{
+    constexpr int WM = 2, WN = 4, TM = 4, TN = 2, NWAVES = 8;
+    constexpr int BM = 256, BN = 256, BK = 32, NS = 4;
+    constexpr int STAGE_BYTES = BM * BK * 2;             // 16 KiB per operand and stage
+    constexpr int ISSUES = BM * 4 / 512;                  // 16-byte chunks per thread, operand and tile (= 2)
+
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = ntiles / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    uint32_t tm, tn;
+    {
+        constexpr uint32_t GM = 8;
+        const uint32_t group = bid / (GM * tiles_n);
+        const uint32_t first = group * GM;
+        const uint32_t rows = tiles_m - first < GM ? tiles_m - first : GM;
+        const uint32_t in = bid - group * GM * tiles_n;
+        tm = first + in % rows;
+        tn = in / rows;
+    }
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // LDS-DMA sources: issue i of a wave fills rows [(i*8 + wave)*16, +16) of the stage
+    const uint16_t *a_src[ISSUES], *w_src[ISSUES];
+    const uint16_t *Wg = reinterpret_cast<const uint16_t *>(g.L.w);
+#pragma unroll
+    for (int i = 0; i < ISSUES; ++i) {
+        const int row = (i * NWAVES + wave) * 16 + (lane >> 2), pos = lane & 3;
+        const int kc = pos ^ ((row >> 2) & 3);
+        const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+        const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+        a_src[i] = g.A + (size_t)m * K + kc * 8;
+        w_src[i] = Wg + (size_t)n * K + kc * 8;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)smem;
+    uint8_t *smem_b = reinterpret_cast<uint8_t *>(smem);
+
+    auto issue_tile = [&](int stage, uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < ISSUES; ++i) {
+            uint8_t *da = smem_b + stage * STAGE_BYTES + (i * NWAVES + wave) * 1024;
+            uint8_t *dw = smem_b + NS * STAGE_BYTES + stage * STAGE_BYTES + (i * NWAVES + wave) * 1024;
+            __builtin_amdgcn_global_load_lds((const void *)(a_src[i] + k0), (__attribute__((address_space(3))) void *)da, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const void *)(w_src[i] + k0), (__attribute__((address_space(3))) void *)dw, 16, 0, 0);
+        }
+    };
+
+    // fragment addresses: k-step ks (0,1), half h -> logical chunk 2ks+h
+    const int h = lane >> 5, sw = (lane >> 2) & 3;
+    uint32_t va[2], vw[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const uint32_t xo = (uint32_t)(((2 * ks + h) ^ sw) << 4);
+        va[ks] = lds0 + (uint32_t)((wm * TM * 32 + (lane & 31)) * 64) + xo;
+        vw[ks] = lds0 + (uint32_t)(NS * STAGE_BYTES) + (uint32_t)((wn * TN * 32 + (lane & 31)) * 64) + xo;
+    }
+    u32x4 fa[2][TM], fb[2][TN];
+
+    auto mfma_group = [&](int cs) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[cs][i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[cs][j]));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if constexpr (F16T) {
+                    f16x8 a, b;
+                    __builtin_memcpy(&a, &fa[cs][i], 16);
+                    __builtin_memcpy(&b, &fb[cs][j], 16);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
+                } else {
+                    bf16x8 a, b;
+                    __builtin_memcpy(&a, &fa[cs][i], 16);
+                    __builtin_memcpy(&b, &fb[cs][j], 16);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
+                }
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    const uint32_t ktiles = K / BK;
+    // prologue: tiles 0, 1, 2 in flight; wait for tile 0, request its first fragments
+    issue_tile(0, 0);
+    if (ktiles > 1) issue_tile(1, BK);
+    if (ktiles > 2) issue_tile(2, 2 * BK);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ktiles > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * ISSUES));
+    else if (ktiles > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ISSUES));
+    else asm volatile("s_waitcnt vmcnt(0)");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    frag_reads64<0, TM>(fa[0], va[0]);
+    frag_reads64<0, TN>(fb[0], vw[0]);
+
+    // one stage; ST = kt % 4 is the LDS buffer of tile kt
+    auto stage = [&](auto st_c, uint32_t kt) {
+        constexpr int ST = decltype(st_c)::value;
+        constexpr int NX = (ST + 1) % NS;
+        // second half of this tile
+        frag_reads64<ST * STAGE_BYTES, TM>(fa[1], va[1]);
+        frag_reads64<ST * STAGE_BYTES, TN>(fb[1], vw[1]);
+        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+        mfma_group(0);
+        // tile kt+1 must have landed everywhere: leave only tile kt+2 in flight
+        if (kt + 2 < ktiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ISSUES));
+        else asm volatile("s_waitcnt vmcnt(0)");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 3 < ktiles) issue_tile((ST + 3) % NS, (kt + 3) * BK);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 1 < ktiles) {
+            frag_reads64<NX * STAGE_BYTES, TM>(fa[0], va[0]);
+            frag_reads64<NX * STAGE_BYTES, TN>(fb[0], vw[0]);
+            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)");
+        }
+        mfma_group(1);
+    };
+
+    for (uint32_t kt = 0; kt < ktiles; kt += 4) {
+        stage(std::integral_constant<int, 0>{}, kt);
+        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 1);
+        if (kt + 2 < ktiles) stage(std::integral_constant<int, 2>{}, kt + 2);
+        if (kt + 3 < ktiles) stage(std::integral_constant<int, 3>{}, kt + 3);
+    }
+
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= M) continue;
+                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
+                const size_t o = (size_t)row * N + col;
+                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // FP32 MFMA GEMM for FP32 weights (n > 64): 64 x 64 x 16 tile, 4 waves
 // ---------------------------------------------------------------------------
@@ -736,6 +1495,11 @@ struct sphip_net {
     // workspace, grown on demand
     uint64_t cap_elems = 0;        // capacity of each ping-pong buffer in FP32 elements
     void *buf[2] = {nullptr, nullptr};
+    uint8_t *aq = nullptr;         // digit planes of the current layer input (integer GEMV)
+    float *aq_inv = nullptr;
+    int *aq_dsum = nullptr;
+    uint32_t aq_valid_layer = 0, aq_valid_n = 0;   // which layer input the planes describe (layer-only timing)
+    uint32_t aq_cap_n = 0;
     float *soft_tmp = nullptr;     // FP32 logits of a softmax layer
     uint64_t soft_cap = 0;
     float *layers_buf = nullptr;   // per-layer activations of a KEEP_LAYERS forward
@@ -799,25 +1563,128 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
     }
 }
 
-void launch_gemv(int fmt, const LayerArgs &L, const float *x, float *y, uint32_t n)
+template <int FMT, int MT>
+void launch_gemv_i8_mt(const GemvI8Args &a, uint32_t grid_x, uint32_t threads, size_t lds)
 {
-    switch (fmt) {
+    auto kern = sp_gemv_i8mfma<FMT, MT>;
+    static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024), true);
+    (void)once;
+    kern<<<grid_x, threads, lds, g_stream>>>(a);
+}
+
+// Integer formats with 16-byte aligned rows go to the INT8 matrix cores:
+// one quantise launch for the layer's input, then the GEMV proper.
+template <int FMT>
+bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
+{
+    constexpr int KL = I8Fmt<FMT>::KL;
+    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq || g_gemv_variant == 0) return false;
+    const int need = (int)(n + 3) / 4;
+    const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
+    GemvI8Args a{};
+    a.L = L; a.x = x; a.y = y; a.nb = (int)n;
+    a.aq = net->aq; a.inv = net->aq_inv; a.dsum = net->aq_dsum;
+    // waves of a workgroup: rw row groups (sharing the digit planes) x ks K shares
+    const uint32_t wave_rows = (L.N + 15) / 16;
+    const uint32_t kblocks = (L.K + KL - 1) / KL;
+    const uint32_t blk_bytes = (uint32_t)I8Fmt<FMT>::NMF * 4u * n * 48u;
+    const uint32_t budget = (uint32_t)g_gemv_lds_kib * 1024u;
+    const uint32_t max_waves = MT > 4 ? 4u : 16u;             // register budget of the wide tiles
+    // the planes cost 3 n bytes per column and workgroup, the weights 2 bits-per-code bytes per
+    // column and row group: more row groups per workgroup as n grows or the codes shrink
+    uint32_t rw = (3u * n + (uint32_t)I8Fmt<FMT>::bits - 1) / (uint32_t)I8Fmt<FMT>::bits;
+    rw = rw >= 4 ? 4u : rw >= 2 ? 2u : 1u;
+    while (rw > 1 && wave_rows / rw < 512u) rw >>= 1;          // keep the grid at least twice the chip
+    uint32_t ks = max_waves / rw > 8u ? 8u : max_waves / rw;
+    if (g_gemv_waves) { rw = (uint32_t)g_gemv_waves & 15u; ks = (uint32_t)g_gemv_waves >> 4; }
+    // one fetch group (4 blocks of every K share) must fit the row, the stage budget and one scale chunk
+    while (ks > 1 && (kblocks < 4u * ks || 4u * ks * blk_bytes > budget)) ks >>= 1;
+    const uint32_t group_blocks = 4u * ks;
+    // scale chunk: about 2048 codes, a whole number of fetch groups, and small enough for one LDS stage
+    uint32_t kc_blocks = 2048u / KL;
+    if (kc_blocks > budget / blk_bytes) kc_blocks = budget / blk_bytes;
+    kc_blocks = kc_blocks / group_blocks * group_blocks;
+    if (kc_blocks == 0) kc_blocks = group_blocks;
+    a.kc = kc_blocks * KL;
+    a.nchunks = (kblocks + kc_blocks - 1) / kc_blocks;
+    a.meta_bytes = a.nchunks * n * 16u;
+    if ((uint64_t)kc_blocks * blk_bytes + a.meta_bytes > 156u * 1024u) return false;
+    const uint32_t nblocks = a.nchunks * kc_blocks;
+    // LDS stage: everything if it fits the budget, else whole scale chunks
+    uint32_t stage = nblocks;
+    if ((uint64_t)nblocks * blk_bytes > budget) {
+        stage = (budget / blk_bytes) / kc_blocks * kc_blocks;
+        if (stage == 0) stage = kc_blocks;
+    }
+    a.stage_blocks = stage;
+    a.rw = rw;
+    a.ks = ks;
+    const uint32_t waves = rw * ks;
+    const uint32_t grid = (wave_rows + rw - 1) / rw;
+    size_t lds = (size_t)stage * blk_bytes;
+    const size_t red_bytes = (size_t)waves * MT * 64u * sizeof(float);
+    if (lds < red_bytes) lds = red_bytes;
+    lds += a.meta_bytes;
+    if (!main_only) sp_quant_x<FMT><<<dim3(a.nchunks, n), 256, 0, g_stream>>>(a);
+    switch (MT) {
+    case 1:  launch_gemv_i8_mt<FMT, 1>(a, grid, waves * 64, lds); break;
+    case 2:  launch_gemv_i8_mt<FMT, 2>(a, grid, waves * 64, lds); break;
+    case 3:  launch_gemv_i8_mt<FMT, 3>(a, grid, waves * 64, lds); break;
+    case 4:  launch_gemv_i8_mt<FMT, 4>(a, grid, waves * 64, lds); break;
+    case 6:  launch_gemv_i8_mt<FMT, 6>(a, grid, waves * 64, lds); break;
+    case 8:  launch_gemv_i8_mt<FMT, 8>(a, grid, waves * 64, lds); break;
+    case 12: launch_gemv_i8_mt<FMT, 12>(a, grid, waves * 64, lds); break;
+    default: launch_gemv_i8_mt<FMT, 16>(a, grid, waves * 64, lds); break;
+    }
+    return true;
+}
+
+void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
+{
+    switch (net->prec) {
     case F32:  launch_gemv_fmt<F32>(L, x, y, n); break;
     case F16:  launch_gemv_fmt<F16>(L, x, y, n); break;
     case BF16: launch_gemv_fmt<BF16>(L, x, y, n); break;
-    case I8:   launch_gemv_fmt<I8>(L, x, y, n); break;
-    case I4:   launch_gemv_fmt<I4>(L, x, y, n); break;
-    default:   launch_gemv_fmt<I2>(L, x, y, n); break;
+    case I8:   if (!launch_gemv_i8<I8>(net, L, x, y, n, main_only)) launch_gemv_fmt<I8>(L, x, y, n); break;
+    case I4:   if (!launch_gemv_i8<I4>(net, L, x, y, n, main_only)) launch_gemv_fmt<I4>(L, x, y, n); break;
+    default:   if (!launch_gemv_i8<I2>(net, L, x, y, n, main_only)) launch_gemv_fmt<I2>(L, x, y, n); break;
     }
 }
 
 template <int FMT, bool F16T>
 void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
 {
-    GemmArgs g{L, A, C, M, out_f32};
+    GemmArgs g{L, A, C, M, out_f32, g_dbg};
+    const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
+    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && g_gemm_variant != 0) {
+        constexpr int BM = 256, BN = 256;
+        const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
+        constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
+        if constexpr (FMT == BF16 || FMT == F16) {
+            if (g_gemm_variant == 3) {
+                constexpr size_t lds4 = 2 * 4 * 256 * 32 * sizeof(uint16_t);
+                auto kern = sp_gemm16_pipe<F16T>;
+                static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4), true);
+                (void)once;
+                kern<<<grid, 512, lds4, g_stream>>>(g);
+                return;
+            }
+        }
+        if (g_gemm_variant == 2) {
+            auto kern = sp_gemm16_big<FMT, F16T, 2, 2, 4, 4>;
+            static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            kern<<<grid, 256, lds, g_stream>>>(g);
+        } else {
+            auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
+            static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            kern<<<grid, 512, lds, g_stream>>>(g);
+        }
+        return;
+    }
     constexpr int TM = 2, TN = 2, BM = 64 * TM, BN = 64 * TN;
     const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
-    const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
     else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
 }
@@ -860,6 +1727,17 @@ int reserve(sphip_net *net, uint32_t n, bool keep_layers)
         net->soft_cap = 0;
         HCHECK(hipMalloc((void **)&net->soft_tmp, soft * sizeof(float)));
         net->soft_cap = soft;
+    }
+    if (n <= 64 && net->prec >= I8 && n > net->aq_cap_n) {
+        // digit planes of the integer GEMV: 4 bytes per element (+ padding of the last chunk), one scale per chunk
+        if (net->aq) { HCHECK(hipFree(net->aq)); HCHECK(hipFree(net->aq_inv)); HCHECK(hipFree(net->aq_dsum)); net->aq = nullptr; }
+        net->aq_cap_n = 0;
+        const uint64_t padded = (uint64_t)n * ((uint64_t)net->max_width + 4096u);
+        HCHECK(hipMalloc((void **)&net->aq, padded * 4u));
+        HCHECK(hipMalloc((void **)&net->aq_inv, (padded / 64u + 64u) * sizeof(float)));
+        HCHECK(hipMalloc((void **)&net->aq_dsum, (padded / 64u + 64u) * 4u * sizeof(int)));
+        net->aq_cap_n = n;
+        net->aq_valid_layer = 0;
     }
     if (keep_layers && !net->layers_buf)
         HCHECK(hipMalloc((void **)&net->layers_buf, net->total_neurons * sizeof(float)));
@@ -916,7 +1794,8 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
         const int out_f32 = (reg != R_GEMM16) || is_last || softmax;
         const bool run = !only_layer || only_layer == l;
         if (run) {
-            if (reg == R_GEMV) launch_gemv(net->prec, L, (const float *)in, (float *)main_out, n);
+            if (reg == R_GEMV) launch_gemv(net, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
+            if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
             else if (reg == R_GEMM32) launch_gemm32(L, (const float *)in, (float *)main_out, n);
             else launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32);
         }
@@ -992,6 +1871,9 @@ void sphip_destroy(sphip_net *net)
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
     for (int i = 0; i < 2; ++i) if (net->buf[i]) (void)hipFree(net->buf[i]);
     if (net->soft_tmp) (void)hipFree(net->soft_tmp);
+    if (net->aq) (void)hipFree(net->aq);
+    if (net->aq_inv) (void)hipFree(net->aq_inv);
+    if (net->aq_dsum) (void)hipFree(net->aq_dsum);
     if (net->layers_buf) (void)hipFree(net->layers_buf);
     if (net->stage_x) (void)hipFree(net->stage_x);
     if (net->stage_y) (void)hipFree(net->stage_y);
