@@ -54,6 +54,15 @@ WORKLOADS = {
 }
 
 
+def compute_dtype(prec: int, n: int) -> str:
+    """Arithmetic type of the path taken (not a precision claim about the weights)."""
+    if prec == S.PRECISION_FLOAT32:
+        return "f32"
+    if n <= 64:
+        return "i8 (exact integer digits, f32 accumulate)" if prec >= S.PRECISION_INT8 else "f32"
+    return "bf16" if prec == S.PRECISION_BFLOAT16 else "f16"
+
+
 def array_payload(n: int, prec: int) -> int:
     """Serialized size of an n-element array including its 4-byte scale (Serialize.c:87-193)."""
     if prec == S.PRECISION_FLOAT32:
@@ -160,7 +169,7 @@ def dominant_layer(topo):
 def roofline_for(copies, topo, prec, n, iters):
     """Times the main kernel of the largest layer alone (HIP events on its stream)."""
     l = dominant_layer(topo)
-    S.time_layer(copies, l, n, 2)
+    S.time_layer(copies, l, n, len(copies) + 2)
     ms = S.time_layer(copies, l, n, iters) / iters
     K, N = topo[l - 1], topo[l]
     kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
@@ -241,6 +250,9 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also make one device-to-device copy of the net's arrays (a plain copy kernel of known "
+                         "size, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -254,6 +266,14 @@ def main():
     n = args.batch or max(cfg["batches"])
     head = run_workload(args.workload, [n], args.steps, args.warmup)
     row = head["rows"][0]
+    if args.calibrate_copy:
+        hc = C.c_void_p()
+        if S.lib().sphip_clone(head["copies"][0].h, C.byref(hc)) == 0:
+            S.synchronize()
+            S.lib().sphip_destroy(hc)
+        print(f"calibration copy: {algorithmic_bytes(cfg['topo'], cfg['prec'], 0)} bytes of arrays "
+              f"(largest single copy {max(array_payload(cfg['topo'][l] * cfg['topo'][l + 1], cfg['prec']) - (4 if cfg['prec'] >= S.PRECISION_INT8 else 0) for l in range(len(cfg['topo']) - 1))} bytes)",
+              file=sys.stderr)
     cpu = None
     if not args.no_cpu:
         sample = min(n, 512 if flops_per_sample(cfg["topo"]) > 5e8 else 4096)
@@ -277,7 +297,7 @@ def main():
         "metric": "forward samples/sec per weight format; % peak HBM BW (b=1), % MFMA peak (b>=4K)",
         "value": row["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": row["steps"], "warmup": args.warmup,
         "ms_per_step": row["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"bf16": "bf16", "fp16": "f16", "fp32": "f32"}.get(row["format"], "bf16"),
+        "dtype": compute_dtype(cfg["prec"], n),
         "data": "synthetic (seeded normal weights through the library's serializer, seeded inputs)",
         "config": {"workload": f"{args.workload}: {'->'.join(map(str, cfg['topo']))} {row['format']} weights, batch {n}",
                    "format": row["format"], "batch": n},

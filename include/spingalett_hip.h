@@ -95,7 +95,7 @@ SPHIP_API int  sphip_time_forward(sphip_net *const *nets, int count, const float
 /* Same for the main kernel of one layer only (layer index 1..layers-1). */
 SPHIP_API int  sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer,
                                 uint32_t n, uint32_t flags, int iters, float *ms);
-/* Name of the kernel sphip_time_layer launches for that layer and n. */
+/* Name of the main kernel the most recent sphip_time_layer call launched. */
 SPHIP_API const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n,
                                               uint32_t flags);
 

@@ -76,6 +76,7 @@ int fail_hip(const char *what, hipError_t e)
 
 hipStream_t g_stream = nullptr;
 int g_dbg = 0;
+const char *g_last_kernel = "";   // main kernel of the most recent layer launch
 int g_gemv_variant = 1;     // 0: vector-ALU GEMV only (tuning switch)
 int g_gemv_waves = 0;       // 0: automatic
 int g_gemv_lds_kib = 64;
@@ -1547,6 +1548,7 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
         const int nb = (int)(n - b0 < 8 ? n - b0 : 8);
         const float *xb = x + (size_t)b0 * L.K;
         float *yb = y + (size_t)b0 * L.N;
+        g_last_kernel = aligned ? "sp_gemv" : "sp_gemv_generic";
         if (aligned) {
             constexpr int R = 2;
             const uint32_t waves = (L.N + R - 1) / R, grid = (waves + 3) / 4;
@@ -1625,6 +1627,7 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     const size_t red_bytes = (size_t)waves * MT * 64u * sizeof(float);
     if (lds < red_bytes) lds = red_bytes;
     lds += a.meta_bytes;
+    g_last_kernel = "sp_gemv_i8mfma";
     if (!main_only) sp_quant_x<FMT><<<dim3(a.nchunks, n), 256, 0, g_stream>>>(a);
     switch (MT) {
     case 1:  launch_gemv_i8_mt<FMT, 1>(a, grid, waves * 64, lds); break;
@@ -1660,8 +1663,10 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         constexpr int BM = 256, BN = 256;
         const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
         constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
+        g_last_kernel = "sp_gemm16_big";
         if constexpr (FMT == BF16 || FMT == F16) {
             if (g_gemm_variant == 3) {
+                g_last_kernel = "sp_gemm16_pipe";
                 constexpr size_t lds4 = 2 * 4 * 256 * 32 * sizeof(uint16_t);
                 auto kern = sp_gemm16_pipe<F16T>;
                 static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4), true);
@@ -1683,6 +1688,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         }
         return;
     }
+    g_last_kernel = "sp_gemm16";
     constexpr int TM = 2, TN = 2, BM = 64 * TM, BN = 64 * TN;
     const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
     if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
@@ -1704,6 +1710,7 @@ void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint
 void launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M)
 {
     Gemm32Args g{L, A, C, M};
+    g_last_kernel = "sp_gemm32_f32";
     const uint32_t grid = ((M + 63) / 64) * ((L.N + 63) / 64);
     sp_gemm32_f32<<<grid, 256, 0, g_stream>>>(g);
 }
@@ -2071,12 +2078,9 @@ int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t
 
 const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, uint32_t flags)
 {
+    (void)n; (void)flags;
     if (!net || layer == 0 || layer >= net->layers) return "";
-    switch (pick_regime(net, n, flags)) {
-    case R_GEMV:   return "sp_gemv";
-    case R_GEMM32: return "sp_gemm32_f32";
-    default:       return "sp_gemm16";
-    }
+    return g_last_kernel;
 }
 
 }  // extern "C"
