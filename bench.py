@@ -162,6 +162,15 @@ def time_workload(copies, topo, n, x_host, steps, warmup):
     return wall * 1e3 / steps, ev_ms / steps, y
 
 
+# HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (summaries and calibration factors: profiles/sp_gemm16_big_C4_bf16_b8192.md,
+# profiles/sp_gemv_i8mfma_C3_int4_b1.md).  Keyed by (kernel, [n, N, K]); None when not profiled.
+PROFILED_TRAFFIC = {
+    ("sp_gemm16_big", (8192, 8192, 8192)): (791942 * 2.0 + 187433 * 1.0) * 1024,
+    ("sp_gemv_i8mfma", (1, 16384, 16384)): (66051 * 2.0 + 64 * 1.0) * 1024,
+}
+
+
 def dominant_layer(topo):
     return 1 + int(np.argmax([topo[l] * topo[l + 1] for l in range(len(topo) - 1)]))
 
@@ -173,17 +182,18 @@ def roofline_for(copies, topo, prec, n, iters):
     ms = S.time_layer(copies, l, n, iters) / iters
     K, N = topo[l - 1], topo[l]
     kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
+    traffic = PROFILED_TRAFFIC.get((kernel, (n, N, K)))
     if n <= 64:
         # memory regime: serialized weights + bias of the layer, FP32 inputs and outputs of the layer
         nbytes = array_payload(K * N, prec) + array_payload(N, prec) + 4 * n * (K + N)
         ach = nbytes / (ms * 1e-3)
         return dict(bound="hbm", achieved=ach / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s", frac=ach / HBM_PEAK,
-                    traffic=None, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+                    traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
     fl = 2.0 * n * K * N
     ach = fl / (ms * 1e-3)
     peak = FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK
     return dict(bound="mfma", achieved=ach / 1e12, peak=peak / 1e12, unit="TFLOP/s", frac=ach / peak,
-                traffic=None, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+                traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
 
 
 def cpu_baseline(path, cfg, n_sample, budget_s=12.0):
