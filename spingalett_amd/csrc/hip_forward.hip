@@ -75,12 +75,11 @@ int fail_hip(const char *what, hipError_t e)
     } while (0)
 
 hipStream_t g_stream = nullptr;
-int g_dbg = 0;
 const char *g_last_kernel = "";   // main kernel of the most recent layer launch
 int g_gemv_variant = 1;     // 0: vector-ALU GEMV only (tuning switch)
 int g_gemv_waves = 0;       // 0: automatic
 int g_gemv_lds_kib = 64;
-int g_gemm_variant = 1;     // 0: 128x128 tiles only; 1: 256x256 / 8 waves; 2: 256x256 / 4 waves (tuning switch)
+int g_gemm_variant = 1;     // 0: 128x128 tiles only (tuning switch)
 
 int ensure_stream()
 {
@@ -91,7 +90,6 @@ int ensure_stream()
     HCHECK(hipSetDevice(0));
     HCHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     if (const char *v = getenv("SPHIP_GEMM_VARIANT")) g_gemm_variant = atoi(v);
-    if (const char *v = getenv("SPHIP_DBG")) g_dbg = atoi(v);
     if (const char *v = getenv("SPHIP_GEMV_VARIANT")) g_gemv_variant = atoi(v);
     if (const char *v = getenv("SPHIP_GEMV_WAVES")) g_gemv_waves = atoi(v);
     if (const char *v = getenv("SPHIP_GEMV_LDS")) g_gemv_lds_kib = atoi(v);
@@ -778,7 +776,6 @@ struct GemmArgs {
     void *C;               // [M][N] 16-bit, or FP32 when out_f32
     uint32_t M;
     int out_f32;
-    int dbg;
 };
 
 // (float)q as a 16-bit float; exact for |q| <= 128 in either type
@@ -997,6 +994,14 @@ __device__ __forceinline__ void frag_reads64(u32x4 *dst, uint32_t addr)
     }
 }
 
+// 16 bytes per lane from global memory straight into LDS (wave-contiguous 1 KiB at lds_addr):
+// scalar base + 32-bit lane offset, so issuing it costs no vector-ALU instruction.  The compiler
+// does not track these loads: the caller waits with s_waitcnt vmcnt before the data is read.
+__device__ __forceinline__ void lds_dma16(uint32_t lds_addr, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+
 template <int OFF>
 __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr)
 {
@@ -1078,39 +1083,57 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // per-thread global source of each direct-to-LDS issue (k offset added per tile)
-    const uint16_t *a_src[A_ISSUES];
+    // LDS-DMA sources: a uniform base (advanced per K tile on the scalar unit) plus a fixed 32-bit
+    // byte offset per lane and issue, and LDS destinations derived from a scalar wave index: the main
+    // loop then issues its loads without any vector-ALU instruction, which would otherwise queue
+    // behind the other wave's MFMAs
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    // Only the first wave of each SIMD (waves 0 .. NWAVES/2-1, which the issue arbiter serves first)
+    // issues the loads, for itself and for wave + NWAVES/2: a wave stalls while the address unit takes
+    // its load, and the other wave of the SIMD keeps the MFMA pipe fed meanwhile.
+    constexpr int HALF = NWAVES / 2;
+    constexpr int A_DUTY = 2 * A_ISSUES, W_DUTY = W_DIRECT ? 2 * W_ISSUES : 1;
+    uint32_t a_voff[A_DUTY], w_voff[W_DUTY];
 #pragma unroll
-    for (int i = 0; i < A_ISSUES; ++i) {
-        const int ci = (i * NWAVES + wave) * 64 + lane, row = ci >> 3, pos = ci & 7;
+    for (int d = 0; d < A_DUTY; ++d) {
+        const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+        const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
         const uint32_t m = m0 + row < M ? m0 + row : M - 1;
-        a_src[i] = g.A + (size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3);
+        a_voff[d] = (uint32_t)(((size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
     }
-    const uint16_t *w_src[W_DIRECT ? W_ISSUES : 1];
     if constexpr (W_DIRECT) {
 #pragma unroll
-        for (int i = 0; i < W_ISSUES; ++i) {
-            const int ci = (i * NWAVES + wave) * 64 + lane, row = ci >> 3, pos = ci & 7;
+        for (int d = 0; d < W_DUTY; ++d) {
+            const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+            const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
             const uint32_t n = n0 + row < N ? n0 + row : N - 1;
-            w_src[i] = reinterpret_cast<const uint16_t *>(g.L.w) + (size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3);
+            w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
         }
     }
+    const char *a_base = reinterpret_cast<const char *>(g.A);
+    const char *w_base = reinterpret_cast<const char *>(g.L.w);
     const size_t w_row_bytes = (size_t)K * bits / 8u;
     uint4 rw[W_LOADS];
-
-    auto issue_direct = [&](int buf, uint32_t k0) {
+    const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)As + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
+    const uint32_t lds_w = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)Ws + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
+    const bool loader = wave_s < HALF;
+    // part = -1: the whole tile; 0, 1, 2: the share issued in front of k-step `part` of the running stage
+    auto issue_direct = [&](int buf, uint32_t k0, int part) {
+        if (!loader) return;
+        const char *ab = a_base + (size_t)k0 * 2u, *wb = w_base + (size_t)k0 * 2u;
+        constexpr int TOTAL = A_DUTY + (W_DIRECT ? W_DUTY : 0);
 #pragma unroll
-        for (int i = 0; i < A_ISSUES; ++i) {
-            uint16_t *dst = As + buf * BM * BK + (i * NWAVES + wave) * 512;      // 64 chunks x 8 elements
-            __builtin_amdgcn_global_load_lds((const void *)(a_src[i] + k0),
-                                             (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+        for (int d = 0; d < A_DUTY; ++d) {
+            const int slot = d * 3 / TOTAL;
+            if (part < 0 || part == slot)
+                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), a_voff[d], ab);
         }
         if constexpr (W_DIRECT) {
 #pragma unroll
-            for (int i = 0; i < W_ISSUES; ++i) {
-                uint16_t *dst = Ws + buf * BN * BK + (i * NWAVES + wave) * 512;
-                __builtin_amdgcn_global_load_lds((const void *)(w_src[i] + k0),
-                                                 (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+            for (int d = 0; d < W_DUTY; ++d) {
+                const int slot = (A_DUTY + d) * 3 / TOTAL;
+                if (part < 0 || part == slot)
+                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), w_voff[d], wb);
             }
         }
     };
@@ -1167,10 +1190,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 
     auto stage = [&](auto cur_c, bool more, uint32_t knext) {
         constexpr int CUR = decltype(cur_c)::value;
-        if (more && !(g.dbg & 1)) {
-            issue_direct(CUR ^ 1, knext);
-            load_w_regs(knext);
-        }
+        if (more) load_w_regs(knext);
         frag_reads<CUR * BM * BK * 2, TM>(fa[0], va[0]);
         frag_reads<CUR * BN * BK * 2, TN>(fb[0], vw[0]);
 #pragma unroll
@@ -1179,6 +1199,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             if (ks < 3) {
                 frag_reads<CUR * BM * BK * 2, TM>(fa[cs ^ 1], va[ks + 1]);
                 frag_reads<CUR * BN * BK * 2, TN>(fb[cs ^ 1], vw[ks + 1]);
+                if (more) issue_direct(CUR ^ 1, knext, ks);
                 asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
             } else {
                 asm volatile("s_waitcnt lgkmcnt(0)");
@@ -1188,7 +1209,6 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 #pragma unroll
             for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[cs][j]));
             __builtin_amdgcn_sched_barrier(0);          // keep the MFMA group between its wait and the next reads
-            if (!(g.dbg & 2))
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1208,198 +1228,20 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             __builtin_amdgcn_sched_barrier(0);
         }
         if (more) store_w_regs(CUR ^ 1);
-        __syncthreads();       // next stage has landed (the fence drains the LDS DMA), this one is free again
+        asm volatile("s_waitcnt vmcnt(0)");         // this wave's share of the next stage has landed
+        __syncthreads();                             // ... and everybody's; the current stage is free again
     };
 
     const uint32_t ktiles = K / BK;
-    issue_direct(0, 0);
+    issue_direct(0, 0, -1);
     load_w_regs(0);
     store_w_regs(0);
+    asm volatile("s_waitcnt vmcnt(0)");
     __syncthreads();
     for (uint32_t kt = 0; kt < ktiles; kt += 2) {
         stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, (kt + 1) * BK);
         if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, (kt + 2) * BK);
     }
-
-    const float wscale = g.L.wscale;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
-        if (col >= N) continue;
-        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row >= M) continue;
-                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
-                const size_t o = (size_t)row * N + col;
-                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
-                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
-            }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Streaming variant for 16-bit weights (BF16 / FP16): 256 x 256 tile, BK = 32,
-// four LDS stages, LDS-DMA three tiles ahead.  The memory pipe is never drained:
-// in the middle of stage t each wave waits only until its share of tile t+1 has
-// landed (s_waitcnt vmcnt leaves the younger tile in flight), meets the other
-// waves at one barrier, then queues tile t+3 into the buffer tile t-1 just left
-// and already requests the first fragments of tile t+1.
-// LDS rows hold 32 elements = four 16-byte chunks; chunk c of row r sits at
-// position c ^ ((r >> 2) & 3): the 16 consecutive rows one fragment-read cycle
-// touches (256 bytes = 4 rows of 64 bytes) fall on 16 different 16-byte slots.
-template <bool F16T>
-__global__ __launch_bounds__(512) void sp_gemm16_pipe(const GemmArgs g)
-{
-    constexpr int WM = 2, WN = 4, TM = 4, TN = 2, NWAVES = 8;
-    constexpr int BM = 256, BN = 256, BK = 32, NS = 4;
-    constexpr int STAGE_BYTES = BM * BK * 2;             // 16 KiB per operand and stage
-    constexpr int ISSUES = BM * 4 / 512;                  // 16-byte chunks per thread, operand and tile (= 2)
-
-    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-
-    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
-    const uint32_t ntiles = tiles_m * tiles_n;
-    uint32_t bid = blockIdx.x;
-    {
-        const uint32_t per = ntiles / 8u;
-        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
-    }
-    uint32_t tm, tn;
-    {
-        constexpr uint32_t GM = 8;
-        const uint32_t group = bid / (GM * tiles_n);
-        const uint32_t first = group * GM;
-        const uint32_t rows = tiles_m - first < GM ? tiles_m - first : GM;
-        const uint32_t in = bid - group * GM * tiles_n;
-        tm = first + in % rows;
-        tn = in / rows;
-    }
-    const uint32_t m0 = tm * BM, n0 = tn * BN;
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    // LDS-DMA sources: issue i of a wave fills rows [(i*8 + wave)*16, +16) of the stage
-    const uint16_t *a_src[ISSUES], *w_src[ISSUES];
-    const uint16_t *Wg = reinterpret_cast<const uint16_t *>(g.L.w);
-#pragma unroll
-    for (int i = 0; i < ISSUES; ++i) {
-        const int row = (i * NWAVES + wave) * 16 + (lane >> 2), pos = lane & 3;
-        const int kc = pos ^ ((row >> 2) & 3);
-        const uint32_t m = m0 + row < M ? m0 + row : M - 1;
-        const uint32_t n = n0 + row < N ? n0 + row : N - 1;
-        a_src[i] = g.A + (size_t)m * K + kc * 8;
-        w_src[i] = Wg + (size_t)n * K + kc * 8;
-    }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)smem;
-    uint8_t *smem_b = reinterpret_cast<uint8_t *>(smem);
-
-    auto issue_tile = [&](int stage, uint32_t k0) {
-#pragma unroll
-        for (int i = 0; i < ISSUES; ++i) {
-            uint8_t *da = smem_b + stage * STAGE_BYTES + (i * NWAVES + wave) * 1024;
-            uint8_t *dw = smem_b + NS * STAGE_BYTES + stage * STAGE_BYTES + (i * NWAVES + wave) * 1024;
-            __builtin_amdgcn_global_load_lds((const void *)(a_src[i] + k0), (__attribute__((address_space(3))) void *)da, 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const void *)(w_src[i] + k0), (__attribute__((address_space(3))) void *)dw, 16, 0, 0);
-        }
-    };
-
-    // fragment addresses: k-step ks (0,1), half h -> logical chunk 2ks+h
-    const int h = lane >> 5, sw = (lane >> 2) & 3;
-    uint32_t va[2], vw[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        const uint32_t xo = (uint32_t)(((2 * ks + h) ^ sw) << 4);
-        va[ks] = lds0 + (uint32_t)((wm * TM * 32 + (lane & 31)) * 64) + xo;
-        vw[ks] = lds0 + (uint32_t)(NS * STAGE_BYTES) + (uint32_t)((wn * TN * 32 + (lane & 31)) * 64) + xo;
-    }
-    u32x4 fa[2][TM], fb[2][TN];
-
-    auto mfma_group = [&](int cs) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[cs][i]));
-#pragma unroll
-        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[cs][j]));
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                if constexpr (F16T) {
-                    f16x8 a, b;
-                    __builtin_memcpy(&a, &fa[cs][i], 16);
-                    __builtin_memcpy(&b, &fb[cs][j], 16);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
-                } else {
-                    bf16x8 a, b;
-                    __builtin_memcpy(&a, &fa[cs][i], 16);
-                    __builtin_memcpy(&b, &fb[cs][j], 16);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
-                }
-            }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    const uint32_t ktiles = K / BK;
-    // prologue: tiles 0, 1, 2 in flight; wait for tile 0, request its first fragments
-    issue_tile(0, 0);
-    if (ktiles > 1) issue_tile(1, BK);
-    if (ktiles > 2) issue_tile(2, 2 * BK);
-    __builtin_amdgcn_sched_barrier(0);
-    if (ktiles > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * ISSUES));
-    else if (ktiles > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ISSUES));
-    else asm volatile("s_waitcnt vmcnt(0)");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    frag_reads64<0, TM>(fa[0], va[0]);
-    frag_reads64<0, TN>(fb[0], vw[0]);
-
-    // one stage; ST = kt % 4 is the LDS buffer of tile kt
-    auto stage = [&](auto st_c, uint32_t kt) {
-        constexpr int ST = decltype(st_c)::value;
-        constexpr int NX = (ST + 1) % NS;
-        // second half of this tile
-        frag_reads64<ST * STAGE_BYTES, TM>(fa[1], va[1]);
-        frag_reads64<ST * STAGE_BYTES, TN>(fb[1], vw[1]);
-        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
-        mfma_group(0);
-        // tile kt+1 must have landed everywhere: leave only tile kt+2 in flight
-        if (kt + 2 < ktiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * ISSUES));
-        else asm volatile("s_waitcnt vmcnt(0)");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 3 < ktiles) issue_tile((ST + 3) % NS, (kt + 3) * BK);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 < ktiles) {
-            frag_reads64<NX * STAGE_BYTES, TM>(fa[0], va[0]);
-            frag_reads64<NX * STAGE_BYTES, TN>(fb[0], vw[0]);
-            asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
-        } else {
-            asm volatile("s_waitcnt lgkmcnt(0)");
-        }
-        mfma_group(1);
-    };
-
-    for (uint32_t kt = 0; kt < ktiles; kt += 4) {
-        stage(std::integral_constant<int, 0>{}, kt);
-        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 1);
-        if (kt + 2 < ktiles) stage(std::integral_constant<int, 2>{}, kt + 2);
-        if (kt + 3 < ktiles) stage(std::integral_constant<int, 3>{}, kt + 3);
-    }
-
     const float wscale = g.L.wscale;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -1569,7 +1411,7 @@ template <int FMT, int MT>
 void launch_gemv_i8_mt(const GemvI8Args &a, uint32_t grid_x, uint32_t threads, size_t lds)
 {
     auto kern = sp_gemv_i8mfma<FMT, MT>;
-    static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024), true);
+    static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024), true);
     (void)once;
     kern<<<grid_x, threads, lds, g_stream>>>(a);
 }
@@ -1657,35 +1499,18 @@ void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float
 template <int FMT, bool F16T>
 void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
 {
-    GemmArgs g{L, A, C, M, out_f32, g_dbg};
+    GemmArgs g{L, A, C, M, out_f32};
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
-    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && g_gemm_variant != 0) {
+    const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
+    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && g_gemm_variant != 0) {
         constexpr int BM = 256, BN = 256;
         const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
         constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
         g_last_kernel = "sp_gemm16_big";
-        if constexpr (FMT == BF16 || FMT == F16) {
-            if (g_gemm_variant == 3) {
-                g_last_kernel = "sp_gemm16_pipe";
-                constexpr size_t lds4 = 2 * 4 * 256 * 32 * sizeof(uint16_t);
-                auto kern = sp_gemm16_pipe<F16T>;
-                static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4), true);
-                (void)once;
-                kern<<<grid, 512, lds4, g_stream>>>(g);
-                return;
-            }
-        }
-        if (g_gemm_variant == 2) {
-            auto kern = sp_gemm16_big<FMT, F16T, 2, 2, 4, 4>;
-            static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-            (void)once;
-            kern<<<grid, 256, lds, g_stream>>>(g);
-        } else {
-            auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
-            static bool once = (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-            (void)once;
-            kern<<<grid, 512, lds, g_stream>>>(g);
-        }
+        auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
+        static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+        (void)once;
+        kern<<<grid, 512, lds, g_stream>>>(g);
         return;
     }
     g_last_kernel = "sp_gemm16";
