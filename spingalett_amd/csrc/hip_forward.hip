@@ -466,87 +466,137 @@ struct I8Fmt {
     static constexpr int BIAS = FMT == I8 ? 0 : FMT == I4 ? 8 : 2;
 };
 
-// Quantise kernel: grid (chunks, nb), one workgroup per sample and scale chunk.
-// Output order = the order the A operand is read.  A 64-byte weight segment
-// (block) is spread over 4 lane groups g of 16 bytes = 4 words w; word w holds
-// WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
+// Digits of the WK activations that meet one 32-bit weight word.  X = rint(x * scale);
+// X + 0x808080 written in plain base 256 has the balanced digits of X, each offset by
+// 128: gather the bytes per digit, then flip the top bits.  Byte i of the operand word
+// of MFMA u comes from code i * NMF + u.
+template <int FMT>
+__device__ __forceinline__ void quant_word(const float4 (&v)[I8Fmt<FMT>::WK / 4], float scale,
+                                           uint32_t (&d0)[I8Fmt<FMT>::NMF], uint32_t (&d1)[I8Fmt<FMT>::NMF],
+                                           uint32_t (&d2)[I8Fmt<FMT>::NMF], int &ds0, int &ds1, int &ds2)
+{
+    constexpr int WK = I8Fmt<FMT>::WK, NMF = I8Fmt<FMT>::NMF;
+    uint32_t Xo[WK];
+#pragma unroll
+    for (int c4 = 0; c4 < WK / 4; ++c4) {
+        Xo[4 * c4 + 0] = (uint32_t)((int)rintf(v[c4].x * scale) + 0x808080);
+        Xo[4 * c4 + 1] = (uint32_t)((int)rintf(v[c4].y * scale) + 0x808080);
+        Xo[4 * c4 + 2] = (uint32_t)((int)rintf(v[c4].z * scale) + 0x808080);
+        Xo[4 * c4 + 3] = (uint32_t)((int)rintf(v[c4].w * scale) + 0x808080);
+    }
+#pragma unroll
+    for (int u = 0; u < NMF; ++u) {
+        const uint32_t x0 = Xo[u], x1 = Xo[NMF + u], x2 = Xo[2 * NMF + u], x3 = Xo[3 * NMF + u];
+        const uint32_t lo01 = __builtin_amdgcn_perm(x1, x0, 0x05040100u);   // x0.b0 x0.b1 x1.b0 x1.b1
+        const uint32_t lo23 = __builtin_amdgcn_perm(x3, x2, 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(x1, x0, 0x0c060c02u);   // x0.b2 0 x1.b2 0
+        const uint32_t hi23 = __builtin_amdgcn_perm(x3, x2, 0x0c060c02u);
+        d0[u] = __builtin_amdgcn_perm(lo23, lo01, 0x06040200u) ^ 0x80808080u;
+        d1[u] = __builtin_amdgcn_perm(lo23, lo01, 0x07050301u) ^ 0x80808080u;
+        d2[u] = __builtin_amdgcn_perm(hi23, hi01, 0x06040200u) ^ 0x80808080u;
+        ds0 = __builtin_amdgcn_sdot4((int)d0[u], 0x01010101, ds0, false);
+        ds1 = __builtin_amdgcn_sdot4((int)d1[u], 0x01010101, ds1, false);
+        ds2 = __builtin_amdgcn_sdot4((int)d2[u], 0x01010101, ds2, false);
+    }
+}
+
+// One wave quantises one scale chunk (kc <= 2048 codes starting at code kbase) of up to NS
+// samples (rows xr, xr + K, ...; ns of them are real): every lane fetches its words'
+// activations in one batch of loads, the wave agrees on the largest magnitude per sample, and
+// each lane converts what it holds.
+// A 64-byte weight segment (block) is spread over 4 lane groups g of 16 bytes = 4 words w;
+// word w holds WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
 //   INT8: 4w+i (u = 0)      INT4: 8w + 2i + u      INT2: 16w + 4i + u
-// of the lane group.  Per (block, u, g) the planes are stored as
+// of the lane group.  store(sample, block in chunk, u, g, w, d0, d1, d2) receives the operand
+// words; done(sample, {bits of 2^-p, sum d0, sum d1, sum d2}) the scale record (same in every lane).
+template <int FMT, int NS, class Store, class Done>
+__device__ __forceinline__ void quant_record(const float *xr, uint32_t K, uint32_t kbase, uint32_t kc, int ns,
+                                             int lane, Store store, Done done)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, F4 = WK / 4;
+    constexpr int MAXIT = 2048 / (64 * WK);
+    constexpr uint32_t WPB = KL / WK;                            // words per block (16)
+    const uint32_t iters = kc / (64u * WK);
+    float4 v[NS][MAXIT][F4];
+    float m[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        m[s] = 0.0f;
+        const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+            const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+            const uint32_t kw = kbase + blk * KL + gg * (KL / 4) + w * WK;     // first code of the word
+            const bool valid = (uint32_t)it < iters && kw < K;                  // rows are whole numbers of words
+            const float4 *src = reinterpret_cast<const float4 *>(xs + (valid ? kw : 0u));
+#pragma unroll
+            for (int c = 0; c < F4; ++c) {
+                float4 t = src[c];
+                if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                v[s][it][c] = t;
+                m[s] = fmaxf(m[s], fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+            }
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        if (s >= ns) break;
+        const float amax = wave_max(m[s]);
+        int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
+        if (e < -126) e = -126;
+        int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
+        p = p > 126 ? 126 : p;
+        const bool live = amax > 0.0f && amax < 3.0e38f;         // zero, inf and NaN chunks contribute nothing
+        const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
+        int ds0 = 0, ds1 = 0, ds2 = 0;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            if ((uint32_t)it < iters) {
+                const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+                const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+                uint32_t d0[NMF], d1[NMF], d2[NMF];
+                quant_word<FMT>(v[s][it], scale, d0, d1, d2, ds0, ds1, ds2);
+#pragma unroll
+                for (int u = 0; u < NMF; ++u) store((uint32_t)s, blk, (uint32_t)u, gg, w, d0[u], d1[u], d2[u]);
+            }
+        }
+        ds0 = wave_sum_i(ds0);
+        ds1 = wave_sum_i(ds1);
+        ds2 = wave_sum_i(ds2);
+        done((uint32_t)s, make_int4(live ? (int)((uint32_t)(127 - p) << 23) : 0, ds0, ds1, ds2));
+    }
+}
+
+// Quantise kernel (n > 4): one wave per sample and scale chunk, four to a workgroup.
+// Output order = the order the A operand is read: per (block, u, g) the planes are stored as
 //   [sample][digit 0..2][16 bytes]
 // i.e. 3 bytes per element and sample; the GEMV kernel copies them verbatim.
 template <int FMT>
 __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
 {
     using F = I8Fmt<FMT>;
-    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK;
-    __shared__ float s_red[4];
-    __shared__ int s_sum[3];
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const uint32_t ch = blockIdx.x, s0 = blockIdx.y, K = a.L.K;
-    const uint32_t k0 = ch * a.kc;
-    const uint32_t klen = k0 + a.kc <= K ? a.kc : K - k0;
+    constexpr int KL = F::KL, NMF = F::NMF;
+    const int lane = threadIdx.x & 63;
+    const uint32_t rec = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (rec >= a.nchunks * (uint32_t)a.nb) return;
+    const uint32_t ch = rec / (uint32_t)a.nb, s0 = rec % (uint32_t)a.nb;
     const uint32_t nblk = a.kc / KL;                         // blocks per chunk (last chunk zero-padded)
-    const float *xs = a.x + (size_t)s0 * K + k0;
-
-    float m = 0.0f;
-    for (uint32_t k = t; k < klen; k += 256) m = fmaxf(m, fabsf(xs[k]));
-    m = wave_max(m);
-    if (lane == 0) s_red[wave] = m;
-    if (t < 3) s_sum[t] = 0;
-    __syncthreads();
-    const float amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
-    if (e < -126) e = -126;
-    int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
-    p = p > 126 ? 126 : p;
-    const bool live = amax > 0.0f && amax < 3.0e38f;         // zero, inf and NaN chunks contribute nothing
-    const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
-
-    int ds0 = 0, ds1 = 0, ds2 = 0;
-    const uint32_t nwords = nblk * (KL / WK);                // weight words per chunk row
-    for (uint32_t wi = t; wi < nwords; wi += 256) {
-        const uint32_t blk = wi / (KL / WK), r = wi % (KL / WK), g = r >> 2, w = r & 3u;
-        const uint32_t kw = blk * KL + g * (KL / 4) + w * WK;      // first code of this word
-        uint32_t d0w[NMF], d1w[NMF], d2w[NMF];
-#pragma unroll
-        for (int u = 0; u < NMF; ++u) d0w[u] = d1w[u] = d2w[u] = 0;
-#pragma unroll
-        for (int c = 0; c < WK; ++c) {
-            const uint32_t k = kw + c;
-            int X = 0;
-            if (k < klen) X = (int)rintf(xs[k] * scale);
-            const int d0 = (int)(int8_t)(X & 255);
-            const int X1 = (X - d0) >> 8;
-            const int d1 = (int)(int8_t)(X1 & 255);
-            const int d2 = (X1 - d1) >> 8;
-            ds0 += d0; ds1 += d1; ds2 += d2;
-            const int u = c % NMF, i = c / NMF;              // code c of the word -> MFMA u, byte i
-            d0w[u] |= (uint32_t)(d0 & 255) << (8 * i);
-            d1w[u] |= (uint32_t)(d1 & 255) << (8 * i);
-            d2w[u] |= (uint32_t)(d2 & 255) << (8 * i);
-        }
-#pragma unroll
-        for (int u = 0; u < NMF; ++u) {
+    quant_record<FMT, 1>(a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, 1, lane,
+        [&](uint32_t, uint32_t blk, uint32_t u, uint32_t g, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
             uint8_t *dst = a.aq + (((((size_t)ch * nblk + blk) * NMF + u) * 4 + g) * (size_t)a.nb + s0) * 48 + w * 4;
-            *reinterpret_cast<uint32_t *>(dst) = d0w[u];
-            *reinterpret_cast<uint32_t *>(dst + 16) = d1w[u];
-            *reinterpret_cast<uint32_t *>(dst + 32) = d2w[u];
-        }
-    }
-    ds0 = wave_sum_i(ds0);
-    ds1 = wave_sum_i(ds1);
-    ds2 = wave_sum_i(ds2);
-    if (lane == 0) {
-        atomicAdd(&s_sum[0], ds0);
-        atomicAdd(&s_sum[1], ds1);
-        atomicAdd(&s_sum[2], ds2);
-    }
-    __syncthreads();
-    if (t == 0) {
-        a.inv[(size_t)ch * a.nb + s0] = live ? __uint_as_float((uint32_t)(127 - p) << 23) : 0.0f;
-        int *d = a.dsum + ((size_t)ch * a.nb + s0) * 4;
-        d[0] = s_sum[0]; d[1] = s_sum[1]; d[2] = s_sum[2]; d[3] = 0;
-    }
+            *reinterpret_cast<uint32_t *>(dst) = d0;
+            *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+            *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+        },
+        [&](uint32_t, int4 md) {
+            if (lane == 0) {
+                a.inv[rec] = __int_as_float(md.x);
+                int *d = a.dsum + (size_t)rec * 4;
+                d[0] = md.y; d[1] = md.z; d[2] = md.w; d[3] = 0;
+            }
+        });
 }
 
 // MT = 16-row A tiles (four samples each).  Rows of D that belong to no sample
@@ -556,8 +606,12 @@ __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
 // rw_id); share ks_id takes the 64-byte blocks ks_id, ks_id + ks, ... of its rows.
 // Weights are fetched in groups of four blocks, the next group in flight while
 // the current one is multiplied; scale chunks are whole numbers of groups.
-template <int FMT, int MT>
-__global__ __launch_bounds__(MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
+//
+// FQ > 0 (n <= FQ <= 4): the workgroup (at most 8 waves) quantises the activations itself,
+// straight into LDS, instead of copying planes a separate launch prepared: every workgroup
+// repeats the (small) job, and the layer costs one launch instead of two.
+template <int FMT, int MT, int FQ>
+__global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
 {
     using F = I8Fmt<FMT>;
     constexpr int KL = F::KL, NMF = F::NMF, G = 4;
@@ -662,19 +716,38 @@ __global__ __launch_bounds__(MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const Gem
     for (int u = 0; u < G; ++u) nxt[u] = load_blk((uint32_t)u);
 
     // scale records of all chunks
-    for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
-        const int *d = a.dsum + (size_t)i * 4;
-        meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
+    if constexpr (!FQ) {
+        for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
+            const int *d = a.dsum + (size_t)i * 4;
+            meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
+        }
     }
 
     uint32_t q = 0;                                            // this wave's block counter
     for (uint32_t ch0 = 0; ch0 < a.nchunks; ch0 += chunks_per_stage) {
         const uint32_t nch = ch0 + chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks - ch0;
         if (ch0) __syncthreads();                             // previous stage fully consumed
-        {
+        if constexpr (!FQ) {
             const uint4 *src = reinterpret_cast<const uint4 *>(a.aq + (size_t)ch0 * kcb * blk_bytes);
             const uint32_t pieces = nch * kcb * (blk_bytes / 16u);
             for (uint32_t i = t; i < pieces; i += nthreads) reinterpret_cast<uint4 *>(A_lds)[i] = src[i];
+        } else {
+            // every wave takes whole scale chunks of this stage, FQ samples at once
+            const uint32_t spc = ((uint32_t)nb + FQ - 1) / FQ;  // sample groups per chunk
+            for (uint32_t ui = (uint32_t)wave; ui < nch * spc; ui += nthreads / 64u) {
+                const uint32_t chl = ui / spc, sbase = (ui % spc) * FQ;
+                const int ns = nb - (int)sbase < FQ ? nb - (int)sbase : FQ;
+                quant_record<FMT, FQ>(a.x + (size_t)sbase * K, K, (ch0 + chl) * a.kc, a.kc, ns, lane,
+                    [&](uint32_t s, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+                        uint8_t *dst = A_lds + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + sbase + s) * 48 + w * 4;
+                        *reinterpret_cast<uint32_t *>(dst) = d0;
+                        *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+                        *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+                    },
+                    [&](uint32_t s, int4 md) {
+                        if (lane == 0) meta[(size_t)(ch0 + chl) * nb + sbase + s] = md;
+                    });
+            }
         }
         __syncthreads();
         const uint8_t *rec = A_lds + (size_t)ks_id * blk_bytes;
@@ -731,6 +804,41 @@ __global__ __launch_bounds__(256) void sp_softmax_rows(const float *__restrict__
     const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (row >= rows) return;
     const float *p = in + (size_t)row * width;
+    auto put = [&](uint32_t i, float v) {
+        const size_t o = (size_t)row * width + i;
+        if (out_kind == 0) reinterpret_cast<float *>(out)[o] = v;
+        else if (out_kind == 1) reinterpret_cast<uint16_t *>(out)[o] = f32_to_bf16_rne(v);
+        else reinterpret_cast<uint16_t *>(out)[o] = f32_to_f16_sat(v);
+    };
+    constexpr int R = 16;                       // rows up to 1024 wide stay in registers: one batch of loads
+    if (width <= (uint32_t)R * kWave) {
+        float v[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint32_t i = (uint32_t)j * kWave + (uint32_t)lane;
+            const float t = p[i < width ? i : 0u];
+            v[j] = i < width ? t : -3.402823466e+38f;
+        }
+        float m = v[0];
+#pragma unroll
+        for (int j = 1; j < R; ++j) m = fmaxf(m, v[j]);
+        m = wave_max(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint32_t i = (uint32_t)j * kWave + (uint32_t)lane;
+            v[j] = i < width ? expf(v[j] - m) : 0.0f;
+            s += v[j];
+        }
+        s = wave_sum(s);
+        const float inv = s > 0.0f ? 1.0f / s : 1.0f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint32_t i = (uint32_t)j * kWave + (uint32_t)lane;
+            if (i < width) put(i, v[j] * inv);
+        }
+        return;
+    }
     float m = -3.402823466e+38f;
     for (uint32_t i = lane; i < width; i += kWave) m = fmaxf(m, p[i]);
     m = wave_max(m);
@@ -738,13 +846,7 @@ __global__ __launch_bounds__(256) void sp_softmax_rows(const float *__restrict__
     for (uint32_t i = lane; i < width; i += kWave) s += expf(p[i] - m);
     s = wave_sum(s);
     const float inv = s > 0.0f ? 1.0f / s : 1.0f;
-    for (uint32_t i = lane; i < width; i += kWave) {
-        const float v = expf(p[i] - m) * inv;
-        const size_t o = (size_t)row * width + i;
-        if (out_kind == 0) reinterpret_cast<float *>(out)[o] = v;
-        else if (out_kind == 1) reinterpret_cast<uint16_t *>(out)[o] = f32_to_bf16_rne(v);
-        else reinterpret_cast<uint16_t *>(out)[o] = f32_to_f16_sat(v);
-    }
+    for (uint32_t i = lane; i < width; i += kWave) put(i, expf(p[i] - m) * inv);
 }
 
 // FP32 -> 16-bit activations for the first GEMM layer
@@ -1407,10 +1509,10 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
     }
 }
 
-template <int FMT, int MT>
+template <int FMT, int MT, int FQ = 0>
 void launch_gemv_i8_mt(const GemvI8Args &a, uint32_t grid_x, uint32_t threads, size_t lds)
 {
-    auto kern = sp_gemv_i8mfma<FMT, MT>;
+    auto kern = sp_gemv_i8mfma<FMT, MT, FQ>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024), true);
     (void)once;
     kern<<<grid_x, threads, lds, g_stream>>>(a);
@@ -1423,6 +1525,7 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
 {
     constexpr int KL = I8Fmt<FMT>::KL;
     if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq || g_gemv_variant == 0) return false;
+    if (reinterpret_cast<uintptr_t>(x) & 15u) return false;   // the quantiser reads float4
     const int need = (int)(n + 3) / 4;
     const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
     GemvI8Args a{};
@@ -1434,13 +1537,33 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     const uint32_t blk_bytes = (uint32_t)I8Fmt<FMT>::NMF * 4u * n * 48u;
     const uint32_t budget = (uint32_t)g_gemv_lds_kib * 1024u;
     const uint32_t max_waves = MT > 4 ? 4u : 16u;             // register budget of the wide tiles
-    // the planes cost 3 n bytes per column and workgroup, the weights 2 bits-per-code bytes per
-    // column and row group: more row groups per workgroup as n grows or the codes shrink
-    uint32_t rw = (3u * n + (uint32_t)I8Fmt<FMT>::bits - 1) / (uint32_t)I8Fmt<FMT>::bits;
-    rw = rw >= 4 ? 4u : rw >= 2 ? 2u : 1u;
-    while (rw > 1 && wave_rows / rw < 512u) rw >>= 1;          // keep the grid at least twice the chip
-    uint32_t ks = max_waves / rw > 8u ? 8u : max_waves / rw;
-    if (g_gemv_waves) { rw = (uint32_t)g_gemv_waves & 15u; ks = (uint32_t)g_gemv_waves >> 4; }
+    // up to four samples: the GEMV workgroups quantise the activations themselves
+    const bool fused = MT == 1 && g_gemv_variant != 2;
+    const uint32_t ks_cap = 2048u / (4u * KL);                 // a scale chunk is a whole number of fetch groups
+                                                               // and at most 2048 codes (one wave's batch of loads)
+    uint32_t rw, ks;
+    if (fused) {
+        // about eight waves per compute unit in all; eight-wave workgroups unless that leaves fewer
+        // workgroups than compute units
+        ks = 2048u / wave_rows;
+        ks = ks >= 8u ? 8u : ks >= 4u ? 4u : ks >= 2u ? 2u : 1u;
+        if (ks > ks_cap) ks = ks_cap;
+        rw = 8u / ks;
+        while (rw > 1 && wave_rows / rw < 256u) rw >>= 1;
+    } else {
+        // the planes cost 3 n bytes per column and workgroup, the weights 2 bits-per-code bytes per
+        // column and row group: more row groups per workgroup as n grows or the codes shrink
+        rw = (3u * n + (uint32_t)I8Fmt<FMT>::bits - 1) / (uint32_t)I8Fmt<FMT>::bits;
+        rw = rw >= 4 ? 4u : rw >= 2 ? 2u : 1u;
+        while (rw > 1 && wave_rows / rw < 512u) rw >>= 1;      // keep the grid at least twice the chip
+        ks = max_waves / rw > 8u ? 8u : max_waves / rw;
+        if (ks > ks_cap) ks = ks_cap;
+    }
+    if (g_gemv_waves) {
+        rw = (uint32_t)g_gemv_waves & 15u; ks = (uint32_t)g_gemv_waves >> 4;
+        if (ks > ks_cap) ks = ks_cap;
+        while (fused && rw * ks > 8u) rw >>= 1;
+    }
     // one fetch group (4 blocks of every K share) must fit the row, the stage budget and one scale chunk
     while (ks > 1 && (kblocks < 4u * ks || 4u * ks * blk_bytes > budget)) ks >>= 1;
     const uint32_t group_blocks = 4u * ks;
@@ -1470,7 +1593,17 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     if (lds < red_bytes) lds = red_bytes;
     lds += a.meta_bytes;
     g_last_kernel = "sp_gemv_i8mfma";
-    if (!main_only) sp_quant_x<FMT><<<dim3(a.nchunks, n), 256, 0, g_stream>>>(a);
+    if (fused) {
+        // samples one wave quantises at once: as many as still leave every wave a unit of work
+        const uint32_t cps = stage / kc_blocks;
+        uint32_t ns = 4;
+        while (ns > 1 && (ns / 2 >= n || cps * ((n + ns - 1) / ns) < waves)) ns >>= 1;
+        if (ns == 1) launch_gemv_i8_mt<FMT, 1, 1>(a, grid, waves * 64, lds);
+        else if (ns == 2) launch_gemv_i8_mt<FMT, 1, 2>(a, grid, waves * 64, lds);
+        else launch_gemv_i8_mt<FMT, 1, 4>(a, grid, waves * 64, lds);
+        return true;
+    }
+    if (!main_only) sp_quant_x<FMT><<<(a.nchunks * n + 3u) / 4u, 256, 0, g_stream>>>(a);
     switch (MT) {
     case 1:  launch_gemv_i8_mt<FMT, 1>(a, grid, waves * 64, lds); break;
     case 2:  launch_gemv_i8_mt<FMT, 2>(a, grid, waves * 64, lds); break;
