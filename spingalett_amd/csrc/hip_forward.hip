@@ -1366,6 +1366,307 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 }
 
 // ---------------------------------------------------------------------------
+// Streaming MFMA kernel for layers with one thin side
+// ---------------------------------------------------------------------------
+// Few samples (5 .. 256) or few outputs (<= 64): one operand is a tall matrix that is
+// read exactly once (the weights, or the 16-bit activations when the layer has few
+// outputs), the other a thin 16-bit matrix of at most 64 rows per workgroup.  The tall
+// operand never touches LDS: a wave owns RT tiles of 32 streamed rows and loads them
+// straight into registers, 16 bytes per lane, one chunk ahead; lanes 0-31 and 32-63 take
+// adjacent 16-byte pieces of a row.  The integer codes become FP16 pairs with the
+// 0x6400 | code trick (1024 + code, minus the constant, exact), which delivers the codes
+// of a step in a format-specific order; the thin operand is written to LDS in that same
+// order, so both MFMA operands agree on which k sits where.
+// Workgroups split K (grid y) to fill the chip; partial tiles go to a workspace and a
+// second launch adds them, otherwise the epilogue is applied here.
+struct SkinnyArgs {
+    LayerArgs L;
+    const uint8_t *stream;   // streamed rows, K codes each
+    const uint16_t *thin;    // [NC][K] 16-bit
+    void *C;                 // [M][N]
+    float *ws;               // [S][NC][R] partial sums when the grid splits K
+    uint32_t R, NC;          // streamed rows, thin rows
+    uint32_t kper;           // codes per K split (whole chunks)
+    int out_f32;
+    int mode_b;              // 0: streamed rows are outputs, thin rows samples; 1: the reverse
+};
+
+template <int FMT>
+struct SkinnyFmt {
+    static constexpr int bits = fmt_bits(FMT);
+    static constexpr int EPL = 128 / bits;                                  // codes per 16-byte lane load
+    static constexpr int LPC = (FMT == I2) ? 2 : 4;                         // lane loads per chunk and tile
+    static constexpr int BKC = 2 * LPC * EPL;                               // codes per chunk: 64 (16-bit), 128, 256, 256
+    static constexpr int STEPS = EPL / 8;                                   // MFMA k-steps per lane load
+    static constexpr int PITCH = BKC * 2 + 16;                              // LDS row pitch: 16 rows hit 16 different slots
+};
+
+// position p of a 16-code group holds code skinny_perm(p) of the group
+template <int FMT>
+__host__ __device__ constexpr int skinny_perm(int p)
+{
+    if (FMT == I8) { constexpr int t[8] = {0, 2, 1, 3, 4, 6, 5, 7}; return t[p & 7] + (p & 8); }
+    if (FMT == I4) { constexpr int t[8] = {0, 4, 1, 5, 2, 6, 3, 7}; return t[p & 7] + (p & 8); }
+    if (FMT == I2) { constexpr int t[16] = {0, 8, 1, 9, 2, 10, 3, 11, 4, 12, 5, 13, 6, 14, 7, 15}; return t[p]; }
+    return p;
+}
+
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t magic_sub(uint32_t v, uint32_t c)
+{
+    h16x2 a, b;
+    __builtin_memcpy(&a, &v, 4);
+    __builtin_memcpy(&b, &c, 4);
+    a = a - b;
+    uint32_t r;
+    __builtin_memcpy(&r, &a, 4);
+    return r;
+}
+
+// The 8 values of k-step j of one lane load, as four FP16 pairs.  A field of the word is
+// masked in place and XORed onto an FP16 constant whose last mantissa bit has the weight of
+// the field's lowest bit (1024 for bit 0, 256 for bit 2, 64 for bit 4, ...), the same XOR flips
+// the field's sign bit (two's complement -> offset binary); subtracting the constant plus the
+// offset leaves the code, exactly.  Only fields above the 10 mantissa bits need a shift first.
+template <int FMT>
+__device__ __forceinline__ void skinny_frag(const uint4 &v, int j, uint32_t (&f)[4])
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (FMT == I8) {
+        // word = codes b0 b1 b2 b3: pairs (b0, b2) and (b1, b3)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t x = w[2 * j + q];
+            f[2 * q]     = magic_sub((x & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);          // 1024 + 128 + q
+            f[2 * q + 1] = magic_sub(((x >> 8) & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);
+        }
+    } else if constexpr (FMT == I4) {
+        // word = nibbles c0 .. c7: pairs (c0, c4), (c1, c5), (c2, c6), (c3, c7)
+        const uint32_t x = w[j], y = x >> 8;
+        f[0] = magic_sub((x & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);                      // 1024 + 8 + q
+        f[1] = magic_sub((x & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);                      // 64 + 8 + q
+        f[2] = magic_sub((y & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);
+        f[3] = magic_sub((y & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);
+    } else if constexpr (FMT == I2) {
+        // word = fields c0 .. c15: step 0 pairs (c0, c8) .. (c3, c11), step 1 pairs (c4, c12) .. (c7, c15)
+        const uint32_t x = w[j >> 1];
+        if ((j & 1) == 0) {
+            f[0] = magic_sub((x & 0x00030003u) ^ 0x64026402u, 0x64026402u);                  // 1024 + 2 + q
+            f[1] = magic_sub((x & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);                  // 256 + 2 + q
+            f[2] = magic_sub((x & 0x00300030u) ^ 0x54205420u, 0x54205420u);                  // 64 + 2 + q
+            f[3] = magic_sub((x & 0x00C000C0u) ^ 0x4C804C80u, 0x4C804C80u);                  // 16 + 2 + q
+        } else {
+            const uint32_t y = x >> 10;
+            f[0] = magic_sub((x & 0x03000300u) ^ 0x46004600u, 0x46004600u);                  // 4 + 2 + q
+            f[1] = magic_sub((y & 0x00030003u) ^ 0x64026402u, 0x64026402u);
+            f[2] = magic_sub((y & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);
+            f[3] = magic_sub((y & 0x00300030u) ^ 0x54205420u, 0x54205420u);
+        }
+    } else {
+        f[0] = w[0]; f[1] = w[1]; f[2] = w[2]; f[3] = w[3];
+    }
+}
+
+template <bool F16T>
+__device__ __forceinline__ void skinny_emit(const SkinnyArgs &a, uint32_t c, uint32_t r, float accv)
+{
+    const uint32_t m = a.mode_b ? r : c, n = a.mode_b ? c : r;
+    const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, n) * a.L.bscale;
+    const float v = apply_act(fmaf(accv, a.L.wscale, bias), a.L.act);
+    const size_t o = (size_t)m * a.L.N + n;
+    if (a.out_f32) reinterpret_cast<float *>(a.C)[o] = v;
+    else reinterpret_cast<uint16_t *>(a.C)[o] = f32_to_t16<F16T>(v);
+}
+
+template <int FMT, bool F16T, int RT, int CT>
+__global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
+{
+    using F = SkinnyFmt<FMT>;
+    constexpr int EPL = F::EPL, LPC = F::LPC, BKC = F::BKC, STEPS = F::STEPS, PITCH = F::PITCH;
+    constexpr int UNITS = 32 * CT * (BKC / 16);            // 16-code units of a thin chunk
+    constexpr int UPT = (UNITS + 255) / 256;
+    constexpr int STAGE = 32 * CT * PITCH;
+    extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t n31 = lane & 31, h = lane >> 5;
+    const uint32_t K = a.L.K;
+    const uint32_t row0 = (blockIdx.x * 4u + (uint32_t)wave) * (32u * RT);
+    const uint32_t cbase = blockIdx.z * (32u * CT);
+    const uint32_t kbeg = blockIdx.y * a.kper;
+    const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
+    const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
+    const size_t row_bytes = (size_t)K * F::bits / 8u;
+
+    const uint8_t *srow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const uint32_t r = row0 + rt * 32u + n31;
+        srow[rt] = a.stream + (size_t)(r < a.R ? r : a.R - 1) * row_bytes;
+    }
+
+    f32x16 acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rt][ct][r] = 0.0f;
+
+    auto load_stream = [&](uint32_t kc0, uint4 (&dst)[RT][LPC]) {
+#pragma unroll
+        for (int i = 0; i < LPC; ++i) {
+            const uint32_t k = kc0 + (2u * i + h) * EPL;            // first code of this lane load
+            const bool valid = k < K;                                // rows are whole numbers of lane loads
+            const size_t off = (size_t)(valid ? k : 0u) * F::bits / 8u;
+            // integer codes past the end of a row meet zeros of the thin operand; 16-bit values there
+            // could be NaN or infinite and are masked
+            const uint32_t keep = (F::bits == 16 && !valid) ? 0u : 0xFFFFFFFFu;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                uint4 v = *reinterpret_cast<const uint4 *>(srow[rt] + off);
+                if constexpr (F::bits == 16) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
+                dst[rt][i] = v;
+            }
+        }
+    };
+    auto load_thin = [&](uint32_t kc0, uint4 (&dst)[UPT][2]) {
+#pragma unroll
+        for (int q = 0; q < UPT; ++q) {
+            const uint32_t u = (uint32_t)t + 256u * q;
+            const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
+            const uint32_t k = kc0 + uc * 16u;
+            const uint32_t c = cbase + row;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const bool valid = u < (uint32_t)UNITS && c < a.NC && k + 8u * e + 8u <= kend;
+                const uint16_t *src = a.thin + (valid ? (size_t)c * K + k + 8u * e : 0u);
+                const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;
+                uint4 v = *reinterpret_cast<const uint4 *>(src);
+                v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
+                dst[q][e] = v;
+            }
+        }
+    };
+    auto store_thin = [&](int stage, const uint4 (&src)[UPT][2]) {
+#pragma unroll
+        for (int q = 0; q < UPT; ++q) {
+            const uint32_t u = (uint32_t)t + 256u * q;
+            if (u >= (uint32_t)UNITS) continue;
+            const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
+            const uint32_t in[8] = {src[q][0].x, src[q][0].y, src[q][0].z, src[q][0].w,
+                                    src[q][1].x, src[q][1].y, src[q][1].z, src[q][1].w};
+            uint32_t o[8];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                constexpr int dummy = 0; (void)dummy;
+                const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
+                const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
+                                     ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
+                o[w] = __builtin_amdgcn_perm(in[eb >> 1], in[ea >> 1], sel);
+            }
+            uint8_t *dst = sk_lds + stage * STAGE + row * PITCH + uc * 32u;
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+        }
+    };
+
+    auto compute = [&](int stage, const uint4 (&cur)[RT][LPC]) {
+        const uint8_t *sbase = sk_lds + stage * STAGE + n31 * PITCH + h * (EPL * 2);
+#pragma unroll
+        for (int i = 0; i < LPC; ++i) {
+#pragma unroll
+            for (int j = 0; j < STEPS; ++j) {
+                constexpr int dummy = 0; (void)dummy;
+                const int koff = (2 * i * EPL + 8 * j) * 2;
+                uint4 tf[CT];
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) tf[ct] = *reinterpret_cast<const uint4 *>(sbase + ct * 32 * PITCH + koff);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    uint32_t sf[4];
+                    skinny_frag<FMT>(cur[rt][i], j, sf);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        if constexpr (F16T) {
+                            f16x8 af, bf;
+                            __builtin_memcpy(&af, &tf[ct], 16);
+                            __builtin_memcpy(&bf, sf, 16);
+                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[rt][ct], 0, 0, 0);
+                        } else {
+                            bf16x8 af, bf;
+                            __builtin_memcpy(&af, &tf[ct], 16);
+                            __builtin_memcpy(&bf, sf, 16);
+                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf, acc[rt][ct], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+    };
+    // one chunk: fetch chunk ch + 1 into `nxt`, multiply chunk ch held in `cur`
+    uint4 thin_regs[UPT][2];
+    auto step = [&](uint32_t ch, const uint4 (&cur)[RT][LPC], uint4 (&nxt)[RT][LPC]) {
+        const int stage = (int)(ch & 1u);
+        const bool more = ch + 1 < nchunks;
+        if (more) {
+            load_stream(kbeg + (ch + 1) * BKC, nxt);
+            load_thin(kbeg + (ch + 1) * BKC, thin_regs);
+        }
+        compute(stage, cur);
+        if (more) store_thin(stage ^ 1, thin_regs);
+        __syncthreads();
+    };
+
+    uint4 ra[RT][LPC], rb[RT][LPC];
+    load_stream(kbeg, ra);
+    load_thin(kbeg, thin_regs);
+    store_thin(0, thin_regs);
+    __syncthreads();
+    for (uint32_t ch = 0; ch < nchunks; ch += 2) {
+        step(ch, ra, rb);
+        if (ch + 1 < nchunks) step(ch + 1, rb, ra);
+    }
+
+    // accumulator register r of lane (n31, h): thin row 8 (r / 4) + 4 h + r % 4, streamed row n31
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const uint32_t r = row0 + rt * 32u + n31;
+        if (r >= a.R) continue;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const uint32_t c = cbase + ct * 32u + 8u * (q >> 2) + 4u * h + (q & 3);
+                if (c >= a.NC) continue;
+                if (a.ws) a.ws[((size_t)blockIdx.y * a.NC + c) * a.R + r] = acc[rt][ct][q];
+                else skinny_emit<F16T>(a, c, r, acc[rt][ct][q]);
+            }
+    }
+}
+
+// adds the K splits of sp_skinny16 and applies bias and activation
+template <bool F16T>
+__global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint32_t splits)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)a.NC * a.R;
+    if (idx >= total) return;
+    float sum = 0.0f;
+    for (uint32_t sp = 0; sp < splits; ++sp) sum += a.ws[(uint64_t)sp * total + idx];
+    skinny_emit<F16T>(a, (uint32_t)(idx / a.R), (uint32_t)(idx % a.R), sum);
+}
+
+// unscaled integer codes of a small weight array as FP16 (the thin operand of a layer with few outputs)
+template <int FMT>
+__global__ __launch_bounds__(256) void sp_codes16(const uint8_t *__restrict__ codes, uint16_t *__restrict__ out, uint64_t n)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) out[i] = f32_to_f16_sat(elem_value<FMT>(codes, i));
+}
+
+// ---------------------------------------------------------------------------
 // FP32 MFMA GEMM for FP32 weights (n > 64): 64 x 64 x 16 tile, 4 waves
 // ---------------------------------------------------------------------------
 struct Gemm32Args {
@@ -1429,6 +1730,8 @@ struct DevArray {
     uint64_t count = 0;
     float max_val = 0.0f;
     bool uploaded = false;
+    uint16_t *codes16 = nullptr;   // weights of a layer with few outputs: unscaled codes as FP16 (made on demand)
+    bool codes16_valid = false;
 };
 
 struct sphip_net {
@@ -1453,6 +1756,8 @@ struct sphip_net {
     uint64_t stage_x_cap = 0, stage_y_cap = 0;
     uint32_t max_width = 0;
     uint64_t total_neurons = 0;
+    float *split_ws = nullptr;     // partial sums of the K splits of the thin-operand kernel
+    uint64_t split_cap = 0;
 };
 
 namespace {
@@ -1463,8 +1768,8 @@ Regime pick_regime(const sphip_net *net, uint32_t n, uint32_t flags)
 {
     if ((flags & SPHIP_FORCE_GEMV) && n <= 64) return R_GEMV;
     if (flags & SPHIP_FORCE_GEMM) return net->prec == F32 ? R_GEMM32 : R_GEMM16;
-    if (n <= 64) return R_GEMV;
-    return net->prec == F32 ? R_GEMM32 : R_GEMM16;
+    if (net->prec == F32) return n <= 64 ? R_GEMV : R_GEMM32;
+    return n <= 4 ? R_GEMV : R_GEMM16;
 }
 
 LayerArgs make_layer_args(const sphip_net *net, uint32_t l /*1-based layer*/)
@@ -1629,9 +1934,96 @@ void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float
     }
 }
 
-template <int FMT, bool F16T>
-void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
+// What the thin-operand kernel needs beyond the layer itself
+struct ThinCtx {
+    const uint16_t *w16;   // [N][K] 16-bit weights (raw 16-bit formats, or FP16 codes) when N <= 64, else nullptr
+    float *ws;             // split-K workspace
+    uint64_t ws_floats;
+};
+
+struct ThinPlan {
+    bool use;
+    bool mode_b;
+    uint32_t R, NC;        // streamed rows, thin rows
+    int rt, ct;
+    uint32_t splits, kper, row_blocks, cblocks;
+};
+
+// mode_b streams 16-bit activations (fmt = the activation type), mode a the weights
+ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
 {
+    ThinPlan p{};
+    const int wbits = fmt_bits(fmt);
+    if (N <= 64 && K % 8u == 0 && M >= 1) {
+        p.use = true; p.mode_b = true; p.R = M; p.NC = N;
+    } else if (M <= 256 && rows_aligned(fmt, K) && K % 8u == 0) {
+        p.use = true; p.mode_b = false; p.R = N; p.NC = M;
+    } else {
+        return p;
+    }
+    const int sfmt = p.mode_b ? F16 : fmt;
+    const uint32_t bkc = sfmt == I8 ? 128u : (sfmt == I4 || sfmt == I2) ? 256u : 64u;
+    (void)wbits;
+    p.ct = p.NC <= 32 ? 1 : 2;
+    p.cblocks = (p.NC + 32u * p.ct - 1) / (32u * p.ct);
+    p.rt = (p.R + 255u) / 256u * p.cblocks >= 128u ? 2 : 1;
+    p.row_blocks = (p.R + 128u * p.rt - 1) / (128u * p.rt);
+    const uint32_t chunks = (K + bkc - 1) / bkc;
+    const uint32_t wgs = p.row_blocks * p.cblocks;
+    uint32_t splits = (512u + wgs - 1) / wgs;
+    if (splits > 16u) splits = 16u;
+    if (splits > chunks / 2u) splits = chunks / 2u;
+    if (splits < 1u) splits = 1u;
+    const uint32_t cps = (chunks + splits - 1) / splits;
+    p.kper = cps * bkc;
+    p.splits = (chunks + cps - 1) / cps;
+    return p;
+}
+
+template <int SFMT, bool F16T, int RT, int CT>
+void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
+{
+    constexpr size_t lds = 2 * 32 * CT * SkinnyFmt<SFMT>::PITCH;
+    auto kern = sp_skinny16<SFMT, F16T, RT, CT>;
+    static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+    (void)once;
+    kern<<<dim3(p.row_blocks, p.splits, p.cblocks), 256, lds, g_stream>>>(a);
+}
+
+template <int SFMT, bool F16T>
+void launch_thin(SkinnyArgs a, const ThinPlan &p)
+{
+    if (p.splits == 1) a.ws = nullptr;
+    if (p.rt == 2) {
+        if (p.ct == 2) launch_thin_inst<SFMT, F16T, 2, 2>(a, p); else launch_thin_inst<SFMT, F16T, 2, 1>(a, p);
+    } else {
+        if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1>(a, p);
+    }
+    if (p.splits > 1) {
+        const uint64_t total = (uint64_t)a.NC * a.R;
+        sp_skinny_reduce<F16T><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(a, p.splits);
+    }
+}
+
+template <int FMT, bool F16T>
+void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
+{
+    const ThinPlan tp = g_gemm_variant == 4 ? ThinPlan{} : plan_thin(FMT, M, L.N, L.K);
+    if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
+        SkinnyArgs a{};
+        a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
+        g_last_kernel = "sp_skinny16";
+        if (tp.mode_b) {
+            a.stream = reinterpret_cast<const uint8_t *>(A);
+            a.thin = ctx.w16;
+            launch_thin<F16T ? F16 : BF16, F16T>(a, tp);
+        } else {
+            a.stream = L.w;
+            a.thin = A;
+            launch_thin<FMT, F16T>(a, tp);
+        }
+        return;
+    }
     GemmArgs g{L, A, C, M, out_f32};
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
@@ -1653,15 +2045,15 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
 }
 
-void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32)
+void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
 {
     switch (fmt) {
-    case F16:  launch_gemm16_fmt<F16, true>(L, A, C, M, out_f32); break;
-    case BF16: launch_gemm16_fmt<BF16, false>(L, A, C, M, out_f32); break;
+    case F16:  launch_gemm16_fmt<F16, true>(L, A, C, M, out_f32, ctx); break;
+    case BF16: launch_gemm16_fmt<BF16, false>(L, A, C, M, out_f32, ctx); break;
     // integer codes are exact in either 16-bit type; FP16 keeps 11 bits of the activations instead of 8
-    case I8:   launch_gemm16_fmt<I8, true>(L, A, C, M, out_f32); break;
-    case I4:   launch_gemm16_fmt<I4, true>(L, A, C, M, out_f32); break;
-    default:   launch_gemm16_fmt<I2, true>(L, A, C, M, out_f32); break;     // FP32 weights never come here
+    case I8:   launch_gemm16_fmt<I8, true>(L, A, C, M, out_f32, ctx); break;
+    case I4:   launch_gemm16_fmt<I4, true>(L, A, C, M, out_f32, ctx); break;
+    default:   launch_gemm16_fmt<I2, true>(L, A, C, M, out_f32, ctx); break;     // FP32 weights never come here
     }
 }
 
@@ -1706,6 +2098,31 @@ int reserve(sphip_net *net, uint32_t n, bool keep_layers)
     }
     if (keep_layers && !net->layers_buf)
         HCHECK(hipMalloc((void **)&net->layers_buf, net->total_neurons * sizeof(float)));
+    if (net->prec != F32) {
+        // thin-operand kernel: split-K workspace, and FP16 copies of the codes of layers with few outputs
+        uint64_t ws = 0;
+        for (uint32_t l = 1; l < net->layers; ++l) {
+            const ThinPlan tp = plan_thin(net->prec, n, net->topo[l], net->topo[l - 1]);
+            if (!tp.use) continue;
+            if (tp.splits > 1 && (uint64_t)tp.splits * tp.NC * tp.R > ws) ws = (uint64_t)tp.splits * tp.NC * tp.R;
+            DevArray &wa = net->W[l - 1];
+            if (tp.mode_b && net->prec >= I8 && !wa.codes16_valid && wa.uploaded) {
+                if (!wa.codes16) HCHECK(hipMalloc((void **)&wa.codes16, wa.count * sizeof(uint16_t)));
+                const uint32_t grid = (uint32_t)((wa.count + 255) / 256);
+                if (net->prec == I8) sp_codes16<I8><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
+                else if (net->prec == I4) sp_codes16<I4><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
+                else sp_codes16<I2><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
+                HCHECK(hipGetLastError());
+                wa.codes16_valid = true;
+            }
+        }
+        if (ws > net->split_cap) {
+            if (net->split_ws) { HCHECK(hipFree(net->split_ws)); net->split_ws = nullptr; }
+            net->split_cap = 0;
+            HCHECK(hipMalloc((void **)&net->split_ws, ws * sizeof(float)));
+            net->split_cap = ws;
+        }
+    }
     return 0;
 }
 
@@ -1762,7 +2179,15 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
             if (reg == R_GEMV) launch_gemv(net, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
             else if (reg == R_GEMM32) launch_gemm32(L, (const float *)in, (float *)main_out, n);
-            else launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32);
+            else {
+                const DevArray &wa = net->W[l - 1];
+                ThinCtx ctx{};
+                if (net->prec == F16 || net->prec == BF16) ctx.w16 = reinterpret_cast<const uint16_t *>(wa.base);
+                else if (wa.codes16_valid) ctx.w16 = wa.codes16;
+                ctx.ws = net->split_ws;
+                ctx.ws_floats = net->split_cap;
+                launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32, ctx);
+            }
         }
         if (softmax && !only_layer) {
             const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
@@ -1832,8 +2257,9 @@ void sphip_destroy(sphip_net *net)
 {
     if (!net) return;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
-    for (auto &a : net->W) if (a.base) (void)hipFree(a.base);
+    for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); }
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
+    if (net->split_ws) (void)hipFree(net->split_ws);
     for (int i = 0; i < 2; ++i) if (net->buf[i]) (void)hipFree(net->buf[i]);
     if (net->soft_tmp) (void)hipFree(net->soft_tmp);
     if (net->aq) (void)hipFree(net->aq);
@@ -1854,6 +2280,7 @@ int sphip_upload_array(sphip_net *net, uint32_t l, int which, const void *codes,
     HCHECK(hipStreamSynchronize(g_stream));
     a.max_val = max_val;
     a.uploaded = true;
+    a.codes16_valid = false;
     return 0;
 }
 
