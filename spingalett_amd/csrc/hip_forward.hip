@@ -502,27 +502,32 @@ __device__ __forceinline__ void quant_word(const float4 (&v)[I8Fmt<FMT>::WK / 4]
 
 // One wave quantises one scale chunk (kc <= 2048 codes starting at code kbase) of up to NS
 // samples (rows xr, xr + K, ...; ns of them are real): every lane fetches its words'
-// activations in one batch of loads, the wave agrees on the largest magnitude per sample, and
-// each lane converts what it holds.
+// activations in one batch of loads (quant_load), the wave agrees on the largest magnitude per
+// sample, and each lane converts what it holds (quant_finish).
 // A 64-byte weight segment (block) is spread over 4 lane groups g of 16 bytes = 4 words w;
 // word w holds WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
 //   INT8: 4w+i (u = 0)      INT4: 8w + 2i + u      INT2: 16w + 4i + u
 // of the lane group.  store(sample, block in chunk, u, g, w, d0, d1, d2) receives the operand
 // words; done(sample, {bits of 2^-p, sum d0, sum d1, sum d2}) the scale record (same in every lane).
-template <int FMT, int NS, class Store, class Done>
-__device__ __forceinline__ void quant_record(const float *xr, uint32_t K, uint32_t kbase, uint32_t kc, int ns,
-                                             int lane, Store store, Done done)
-{
-    using F = I8Fmt<FMT>;
-    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, F4 = WK / 4;
-    constexpr int MAXIT = 2048 / (64 * WK);
-    constexpr uint32_t WPB = KL / WK;                            // words per block (16)
-    const uint32_t iters = kc / (64u * WK);
+template <int FMT, int NS>
+struct QuantRegs {
+    static constexpr int MAXIT = 2048 / (64 * I8Fmt<FMT>::WK);
+    static constexpr int F4 = I8Fmt<FMT>::WK / 4;
     float4 v[NS][MAXIT][F4];
     float m[NS];
+};
+
+template <int FMT, int NS>
+__device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *xr, uint32_t K, uint32_t kbase,
+                                           uint32_t kc, int ns, int lane)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, WK = F::WK, F4 = WK / 4, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr uint32_t WPB = KL / WK;                            // words per block (16)
+    const uint32_t iters = kc / (64u * WK);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        m[s] = 0.0f;
+        q.m[s] = 0.0f;
         const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
@@ -535,15 +540,24 @@ __device__ __forceinline__ void quant_record(const float *xr, uint32_t K, uint32
             for (int c = 0; c < F4; ++c) {
                 float4 t = src[c];
                 if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                v[s][it][c] = t;
-                m[s] = fmaxf(m[s], fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+                q.v[s][it][c] = t;
+                q.m[s] = fmaxf(q.m[s], fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
             }
         }
     }
+}
+
+template <int FMT, int NS, class Store, class Done>
+__device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32_t kc, int ns, int lane, Store store, Done done)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr uint32_t WPB = KL / WK;
+    const uint32_t iters = kc / (64u * WK);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
         if (s >= ns) break;
-        const float amax = wave_max(m[s]);
+        const float amax = wave_max(q.m[s]);
         int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
         if (e < -126) e = -126;
         int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
@@ -557,7 +571,7 @@ __device__ __forceinline__ void quant_record(const float *xr, uint32_t K, uint32
                 const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
                 const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
                 uint32_t d0[NMF], d1[NMF], d2[NMF];
-                quant_word<FMT>(v[s][it], scale, d0, d1, d2, ds0, ds1, ds2);
+                quant_word<FMT>(q.v[s][it], scale, d0, d1, d2, ds0, ds1, ds2);
 #pragma unroll
                 for (int u = 0; u < NMF; ++u) store((uint32_t)s, blk, (uint32_t)u, gg, w, d0[u], d1[u], d2[u]);
             }
@@ -583,7 +597,9 @@ __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
     if (rec >= a.nchunks * (uint32_t)a.nb) return;
     const uint32_t ch = rec / (uint32_t)a.nb, s0 = rec % (uint32_t)a.nb;
     const uint32_t nblk = a.kc / KL;                         // blocks per chunk (last chunk zero-padded)
-    quant_record<FMT, 1>(a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, 1, lane,
+    QuantRegs<FMT, 1> qr;
+    quant_load<FMT, 1>(qr, a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, 1, lane);
+    quant_finish<FMT, 1>(qr, a.kc, 1, lane,
         [&](uint32_t, uint32_t blk, uint32_t u, uint32_t g, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
             uint8_t *dst = a.aq + (((((size_t)ch * nblk + blk) * NMF + u) * 4 + g) * (size_t)a.nb + s0) * 48 + w * 4;
             *reinterpret_cast<uint32_t *>(dst) = d0;
@@ -710,10 +726,27 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
         }
     };
 
-    // first weight group goes out before anything else
-    uint4 nxt[G];
+    // The self-quantising variant requests the activations of its first scale chunk before the
+    // weights: loads complete in order, and the quantiser should not wait behind the weight stream.
+    constexpr int QN = FQ ? FQ : 1;
+    QuantRegs<FMT, QN> qr;
+    const uint32_t spc = ((uint32_t)nb + QN - 1) / QN;         // sample groups per chunk
+    const uint32_t nch_first = chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks;
+    auto unit_load = [&](uint32_t ch0, uint32_t ui) {
+        const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
+        const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
+        quant_load<FMT, QN>(qr, a.x + (size_t)sbase * K, K, (ch0 + chl) * a.kc, a.kc, ns, lane);
+    };
+    if constexpr (FQ != 0) {
+        if ((uint32_t)wave < nch_first * spc) unit_load(0u, (uint32_t)wave);
+    }
+    // then the first weight group (PD groups in flight; two measured slower than one)
+    constexpr int PD = 1;
+    uint4 nxt[PD][G];
 #pragma unroll
-    for (int u = 0; u < G; ++u) nxt[u] = load_blk((uint32_t)u);
+    for (int d = 0; d < PD; ++d)
+#pragma unroll
+        for (int u = 0; u < G; ++u) nxt[d][u] = load_blk((uint32_t)(d * G + u));
 
     // scale records of all chunks
     if constexpr (!FQ) {
@@ -733,11 +766,11 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
             for (uint32_t i = t; i < pieces; i += nthreads) reinterpret_cast<uint4 *>(A_lds)[i] = src[i];
         } else {
             // every wave takes whole scale chunks of this stage, FQ samples at once
-            const uint32_t spc = ((uint32_t)nb + FQ - 1) / FQ;  // sample groups per chunk
             for (uint32_t ui = (uint32_t)wave; ui < nch * spc; ui += nthreads / 64u) {
-                const uint32_t chl = ui / spc, sbase = (ui % spc) * FQ;
-                const int ns = nb - (int)sbase < FQ ? nb - (int)sbase : FQ;
-                quant_record<FMT, FQ>(a.x + (size_t)sbase * K, K, (ch0 + chl) * a.kc, a.kc, ns, lane,
+                if (ch0 != 0 || ui != (uint32_t)wave) unit_load(ch0, ui);      // the first one is on its way
+                const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
+                const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
+                quant_finish<FMT, QN>(qr, a.kc, ns, lane,
                     [&](uint32_t s, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
                         uint8_t *dst = A_lds + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + sbase + s) * 48 + w * 4;
                         *reinterpret_cast<uint32_t *>(dst) = d0;
@@ -756,10 +789,14 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
             for (uint32_t gi = 0; gi < groups_per_chunk; ++gi) {
                 uint4 cur[G];
 #pragma unroll
-                for (int u = 0; u < G; ++u) cur[u] = nxt[u];
+                for (int u = 0; u < G; ++u) cur[u] = nxt[0][u];
                 q += G;
 #pragma unroll
-                for (int u = 0; u < G; ++u) nxt[u] = load_blk(q + u);
+                for (int d = 0; d + 1 < PD; ++d)
+#pragma unroll
+                    for (int u = 0; u < G; ++u) nxt[d][u] = nxt[d + 1][u];
+#pragma unroll
+                for (int u = 0; u < G; ++u) nxt[PD - 1][u] = load_blk(q + (PD - 1) * G + u);
 #pragma unroll
                 for (int u = 0; u < G; ++u) process(cur[u], rec + (size_t)u * rstep);
                 rec += G * rstep;
