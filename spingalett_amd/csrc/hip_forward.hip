@@ -1123,16 +1123,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int OFF>
 __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
 
-// CNT fragments 2 KiB apart (32 tile rows of 64 bytes) starting at addr + BASE
-template <int BASE, int CNT, int I = 0>
-__device__ __forceinline__ void frag_reads64(u32x4 *dst, uint32_t addr)
-{
-    if constexpr (I < CNT) {
-        ds_read128<BASE + I * 2048>(dst[I], addr);
-        frag_reads64<BASE, CNT, I + 1>(dst, addr);
-    }
-}
-
 // 16 bytes per lane from global memory straight into LDS (wave-contiguous 1 KiB at lds_addr):
 // scalar base + 32-bit lane offset, so issuing it costs no vector-ALU instruction.  The compiler
 // does not track these loads: the caller waits with s_waitcnt vmcnt before the data is read.
@@ -2064,9 +2054,12 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     GemmArgs g{L, A, C, M, out_f32};
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
-    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && g_gemm_variant != 0) {
+    // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
+    const uint32_t big_tiles = ((M + 255u) / 256u) * ((L.N + 255u) / 256u);
+    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && g_gemm_variant != 0 &&
+        (big_tiles >= 192u || g_gemm_variant == 5)) {
         constexpr int BM = 256, BN = 256;
-        const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
+        const uint32_t grid = big_tiles;
         constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
         g_last_kernel = "sp_gemm16_big";
         auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
