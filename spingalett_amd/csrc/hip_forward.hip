@@ -915,6 +915,8 @@ struct GemmArgs {
     void *C;               // [M][N] 16-bit, or FP32 when out_f32
     uint32_t M;
     int out_f32;
+    float *ws;             // [splits][M][N] partial sums when the grid splits K (sp_gemm16_big only), else nullptr
+    uint32_t kper;         // k range of one split, a multiple of 64 (0: all of K)
 };
 
 // (float)q as a 16-bit float; exact for |q| <= 128 in either type
@@ -1361,15 +1363,33 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
         __syncthreads();                             // ... and everybody's; the current stage is free again
     };
 
-    const uint32_t ktiles = K / BK;
-    issue_direct(0, 0, -1);
-    load_w_regs(0);
+    // grid y splits K for problems with too few tiles to fill the chip
+    const uint32_t kbeg = g.kper ? blockIdx.y * g.kper : 0u;
+    const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
+    const uint32_t ktiles = (kend - kbeg) / BK;
+    issue_direct(0, kbeg, -1);
+    load_w_regs(kbeg);
     store_w_regs(0);
     asm volatile("s_waitcnt vmcnt(0)");
     __syncthreads();
     for (uint32_t kt = 0; kt < ktiles; kt += 2) {
-        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, (kt + 1) * BK);
-        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, (kt + 2) * BK);
+        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, kbeg + (kt + 1) * BK);
+        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, kbeg + (kt + 2) * BK);
+    }
+    if (g.ws) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+            if (col >= N) continue;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < M) g.ws[((size_t)blockIdx.y * M + row) * N + col] = acc[i][j][r];
+                }
+        }
+        return;
     }
     const float wscale = g.L.wscale;
 #pragma unroll
@@ -1390,6 +1410,22 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             }
         }
     }
+}
+
+// adds the K splits of sp_gemm16_big (in split order) and applies scale, bias and activation
+template <bool F16T>
+__global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32_t splits)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)g.M * g.L.N;
+    if (idx >= total) return;
+    float sum = 0.0f;
+    for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
+    const uint32_t col = (uint32_t)(idx % g.L.N);
+    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+    const float v = apply_act(fmaf(sum, g.L.wscale, bias), g.L.act);
+    if (g.out_f32) reinterpret_cast<float *>(g.C)[idx] = v;
+    else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
 }
 
 // ---------------------------------------------------------------------------
@@ -2019,6 +2055,21 @@ void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float
     }
 }
 
+// K splits of the 256 x 256 GEMM when its tiles would leave compute units idle: at least eight K tiles each
+uint32_t gemm16_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
+{
+    const uint32_t tiles = ((M + 255u) / 256u) * ((N + 255u) / 256u), ktiles = K / 64u;
+    *kper = 0;
+    if (tiles >= 192u || ktiles < 16u) return 1;
+    uint32_t splits = (256u + tiles - 1) / tiles;
+    if (splits > 8u) splits = 8u;
+    if (splits > ktiles / 8u) splits = ktiles / 8u;
+    if (splits <= 1u) return 1;
+    const uint32_t per = (ktiles + splits - 1) / splits;
+    *kper = per * 64u;
+    return (ktiles + per - 1) / per;
+}
+
 // What the thin-operand kernel needs beyond the layer itself
 struct ThinCtx {
     const uint16_t *w16;   // [N][K] 16-bit weights (raw 16-bit formats, or FP16 codes) when N <= 64, else nullptr
@@ -2109,23 +2160,29 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         }
         return;
     }
-    GemmArgs g{L, A, C, M, out_f32};
+    GemmArgs g{L, A, C, M, out_f32, nullptr, 0};
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
     // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
     const uint32_t big_tiles = ((M + 255u) / 256u) * ((L.N + 255u) / 256u);
+    const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
+    const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats && g_gemm_variant != 7;
     if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && g_gemm_variant != 0 &&
-        (big_tiles >= 192u || g_gemm_variant == 5)) {
+        (big_tiles >= 192u || split_ok || g_gemm_variant == 5)) {
         constexpr int BM = 256, BN = 256;
-        const uint32_t grid = big_tiles;
+        if (big_tiles >= 192u || !split_ok) g.kper = 0;
+        else g.ws = ctx.ws;
+        const dim3 grid(big_tiles, g.ws ? splits : 1u);
         constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
         g_last_kernel = "sp_gemm16_big";
         auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
         static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
         (void)once;
         kern<<<grid, 512, lds, g_stream>>>(g);
+        if (g.ws) sp_gemm16_reduce<F16T><<<(uint32_t)(((uint64_t)M * L.N + 255) / 256), 256, 0, g_stream>>>(g, splits);
         return;
     }
+    g.kper = 0;
     g_last_kernel = "sp_gemm16";
     constexpr int TM = 2, TN = 2, BM = 64 * TM, BN = 64 * TN;
     const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
@@ -2224,7 +2281,12 @@ int reserve(sphip_net *net, uint32_t n, bool keep_layers)
         uint64_t ws = 0;
         for (uint32_t l = 1; l < net->layers; ++l) {
             const ThinPlan tp = plan_thin(net->prec, n, net->topo[l], net->topo[l - 1]);
-            if (!tp.use) continue;
+            if (!tp.use) {
+                uint32_t kper = 0;
+                const uint32_t sp = gemm16_splits(n, net->topo[l], net->topo[l - 1], &kper);
+                if (sp > 1 && (uint64_t)sp * n * net->topo[l] > ws) ws = (uint64_t)sp * n * net->topo[l];
+                continue;
+            }
             if (tp.splits > 1 && (uint64_t)tp.splits * tp.NC * tp.R > ws) ws = (uint64_t)tp.splits * tp.NC * tp.R;
             DevArray &wa = net->W[l - 1];
             if (tp.mode_b && net->prec >= I8 && !wa.codes16_valid && wa.uploaded) {

@@ -241,10 +241,13 @@ def _decoded_layer(S, fmt, N, K, seed):
     # few outputs, activations streamed
     ("i8", 10, 1000, 256), ("i8", 10, 1000, 4096), ("i4", 64, 512, 1000), ("i2", 33, 2048, 513),
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
+    # a few hundred samples: 256 x 256 tiles with K split over the grid
+    ("i4", 1024, 2048, 300), ("bf16", 768, 1024, 513), ("i2", 2048, 4096, 1000), ("f16", 512, 1024, 257), ("i8", 1280, 1536, 600),
 ])
-def test_thin_operand_kernel_shapes(S, fmt, N, K, n):
+def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     """Layers with one thin side (5..256 samples, or at most 64 outputs) run a weight- or
-    activation-streaming MFMA kernel with split K; checked against FP64 on the decoded arrays."""
+    activation-streaming MFMA kernel with split K, mid-size batches the tiled GEMM with split K;
+    checked against FP64 on the decoded arrays."""
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + K + n)
     X = np.random.default_rng(n).standard_normal((n, K)).astype(F32)
     pre = X.astype(np.float64) @ W.T + b
