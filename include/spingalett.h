@@ -213,6 +213,18 @@ SPINGALETT_API int spingalett_forward_batch_device(NeuralNetwork *net, const flo
                                                    uint32_t n, float *d_outputs);
 SPINGALETT_API int spingalett_hip_synchronize(void);
 
+/* Evaluation of a labelled batch on the device: the forward, then what the reference's epoch
+ * loop does with the outputs — compute_sample_loss per sample (SIMD.c:522-552) with the net's
+ * loss_func and output activation, added over the batch (batch_compute_loss, Training.c:421-435)
+ * — plus the index of the largest output per sample.  inputs [n][topology[0]] and targets
+ * [n][topology[last]] are host memory; total_loss receives the sum of the per-sample losses,
+ * predictions (n entries) and correct (samples whose prediction is the index of the target's
+ * largest entry) may be NULL.  Only these results cross PCIe, not the [n][out] outputs.
+ * Returns 0, or 1 with the error slot set. */
+SPINGALETT_API int spingalett_evaluate_batch(NeuralNetwork *net, const float *inputs, const float *targets,
+                                             uint32_t n, float *total_loss, uint32_t *predictions,
+                                             uint32_t *correct);
+
 /* The device copy is made at the first forward and kept.  Call this after
  * writing net->weights / net->biases by hand: the next forward re-uploads
  * from the FP32 host arrays (the packed arrays of a loaded file are dropped,

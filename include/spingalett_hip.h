@@ -62,11 +62,23 @@ SPHIP_API int  sphip_upload_array(sphip_net *net, uint32_t l, int which,
 /* Replaces forward_struct_arguments (Network.c:202-251) for n = 1 and
  * batch_forward (Training.c:313-345) for n > 1:
  *   per layer  y = act(b + W x), x row-major [n][topology[0]], y row-major
- *   [n][topology[last]], FP32.  n <= 64 runs the vector (GEMV) kernels in
- *   FP32 arithmetic; larger n runs the matrix-core kernels with 16-bit
- *   activations (FP32 weights always use FP32 arithmetic). */
+ *   [n][topology[last]], FP32.  n <= 4 runs the vector (GEMV) kernels in FP32-grade
+ *   arithmetic (integer weights: exact integer dot products on the INT8 matrix
+ *   cores); larger n runs the matrix-core kernels with 16-bit activations.  FP32
+ *   weights always compute in FP32 (vector kernels up to n = 64). */
 SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y,
                              uint32_t flags);
+/* The evaluation step that follows batch_forward in the reference's epoch loop, on the device:
+ * forward of n samples, then per sample compute_sample_loss (SIMD.c:522-552) and the index of
+ * the first largest output, then the batch total (batch_compute_loss, Training.c:421-435;
+ * added in FP64 here).  Only the totals and, when asked for, n indices travel back.
+ *   x, targets  : [n][in], [n][out] FP32; host memory, or both device memory with SPHIP_X_ON_DEVICE
+ *   loss_func   : LossFunction value (Spingalett.h:49-53): 0 squared error, 1 cross-entropy (binary
+ *                 form when the output layer is a sigmoid)
+ *   total_loss  : sum of the per-sample losses;  predictions: [n] host array or NULL;
+ *   correct     : samples whose prediction equals the index of the target's first largest entry, or NULL */
+SPHIP_API int  sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_t n, int loss_func,
+                              uint32_t flags, float *total_loss, uint32_t *predictions, uint32_t *correct);
 /* After a SPHIP_KEEP_LAYERS forward: copies all layers' activations to a host
  * array laid out like NeuralNetwork.neurons (Network.c:16-32). */
 SPHIP_API int  sphip_read_layers(sphip_net *net, float *host_neurons);

@@ -75,6 +75,11 @@ def lib():
     L.orc_forward_batch_f64.argtypes = [P(_Net), C.c_void_p, C.c_uint32, C.c_void_p]
     L.orc_time_forward_batch.restype = C.c_double
     L.orc_time_forward_batch.argtypes = [P(_Net), C.c_void_p, C.c_uint32, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+    L.orc_sample_loss.restype = C.c_float
+    L.orc_sample_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_int, C.c_int]
+    L.orc_batch_loss.restype = C.c_float
+    L.orc_batch_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_int, C.c_int]
+    L.orc_argmax.restype = C.c_uint32; L.orc_argmax.argtypes = [C.c_void_p, C.c_uint32]
     _lib = L
     return L
 
@@ -212,6 +217,23 @@ def activate(x: np.ndarray, act: int) -> np.ndarray:
     y = np.ascontiguousarray(y)
     lib().orc_apply_activation(_ptr(y), y.shape[0], y.shape[1], act)
     return y.reshape(np.shape(x))
+
+
+def sample_loss(output: np.ndarray, target: np.ndarray, loss: int, output_act: int) -> float:
+    o = np.ascontiguousarray(output, dtype=np.float32)
+    t = np.ascontiguousarray(target, dtype=np.float32)
+    return float(lib().orc_sample_loss(_ptr(o), _ptr(t), o.size, loss, output_act))
+
+
+def batch_loss(outputs: np.ndarray, targets: np.ndarray, loss: int, output_act: int) -> float:
+    o = np.ascontiguousarray(outputs, dtype=np.float32)
+    t = np.ascontiguousarray(targets, dtype=np.float32)
+    return float(lib().orc_batch_loss(_ptr(o), _ptr(t), o.shape[0], o.shape[1], loss, output_act))
+
+
+def argmax_rows(outputs: np.ndarray) -> np.ndarray:
+    o = np.ascontiguousarray(outputs, dtype=np.float32)
+    return np.array([lib().orc_argmax(_ptr(o[i]), o.shape[1]) for i in range(o.shape[0])], dtype=np.uint32)
 
 
 # --------------------------------------------------------------------------

@@ -518,6 +518,55 @@ void orc_forward_batch_f64(const orc_net *n, const float *X, uint32_t N, double 
     free(a); free(b);
 }
 
+/* ------------------------------------------------------------------ evaluation */
+/* SIMD.c:522-552 (compute_sample_loss) */
+float orc_sample_loss(const float *output, const float *target, uint32_t width, int loss, int output_act)
+{
+    const float eps = 1e-9f;
+    float acc = 0.0f;
+    if (loss == 0) {
+        for (uint32_t k = 0; k < width; ++k) {
+            const float d = output[k] - target[k];
+            acc += d * d;
+        }
+    } else if (loss == 1) {
+        if (output_act == ORC_ACT_SIGMOID) {
+            for (uint32_t k = 0; k < width; ++k) {
+                float o = output[k];
+                const float t = target[k];
+                if (o < eps) o = eps;
+                if (o > 1.0f - eps) o = 1.0f - eps;
+                acc -= (t * logf(o) + (1.0f - t) * logf(1.0f - o));
+            }
+        } else {
+            for (uint32_t k = 0; k < width; ++k) {
+                float o = output[k];
+                if (o < eps) o = eps;
+                acc -= target[k] * logf(o);
+            }
+        }
+    }
+    return acc;
+}
+
+/* Training.c:421-435 (batch_compute_loss) */
+float orc_batch_loss(const float *outputs, const float *targets, uint32_t N, uint32_t width, int loss, int output_act)
+{
+    float total = 0.0f;
+    for (uint32_t s = 0; s < N; ++s)
+        total += orc_sample_loss(outputs + (size_t)s * width, targets + (size_t)s * width, width, loss, output_act);
+    return total;
+}
+
+uint32_t orc_argmax(const float *row, uint32_t width)
+{
+    uint32_t best = 0;
+    for (uint32_t k = 1; k < width; ++k)
+        if (row[k] > row[best]) best = k;
+    return best;
+}
+
+
 double orc_time_forward_batch(const orc_net *n, const float *X, uint32_t N, float *out,
                               int iters, void *sgemm_fn, int threads)
 {

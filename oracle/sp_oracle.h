@@ -22,6 +22,10 @@
  *   orc_forward_* ........................... pinned: float64 brute force on
  *        small nets, numpy matmul + scipy special functions at size, closed
  *        forms for the piecewise-linear activations, softmax invariants.
+ *   orc_sample_loss / orc_batch_loss ........ pinned: closed forms (MSE of known
+ *        vectors, -log of the target's probability for one-hot targets, the
+ *        1e-9 clamps at 0 and 1, binary cross-entropy symmetry).
+ *   orc_argmax .............................. pinned: numpy argmax (first maximum).
  *   The last-bit summation order of the reference's BLAS / AVX dot product is
  *   deliberately not reproduced (tolerance 1e-4, not bits).
  */
@@ -100,6 +104,17 @@ void orc_forward_single(const orc_net *net, const float *x, float *out);
 void orc_forward_batch(const orc_net *net, const float *X, uint32_t N, float *out);
 /* Same mathematics in float64 end to end (brute-force check, not the reference). */
 void orc_forward_batch_f64(const orc_net *net, const float *X, uint32_t N, double *out);
+
+/* --- evaluation after the batched forward --- */
+/* compute_sample_loss (SIMD.c:522-552): loss 0 = MSE sum of squared differences,
+ * 1 = cross-entropy (-sum t log max(o, 1e-9); with a sigmoid output layer the
+ * binary form with o clamped to [1e-9, 1 - 1e-9]). */
+float orc_sample_loss(const float *output, const float *target, uint32_t width, int loss, int output_act);
+/* batch_compute_loss (Training.c:421-435): the per-sample losses added in sample order, FP32. */
+float orc_batch_loss(const float *outputs, const float *targets, uint32_t N, uint32_t width,
+                     int loss, int output_act);
+/* index of the first largest element of a row (the prediction compared with the label) */
+uint32_t orc_argmax(const float *row, uint32_t width);
 
 /* CPU-baseline leg: same call sequence with a threaded sgemm.  sgemm_fn is a
  * cblas_sgemm-compatible pointer found at run time, or NULL for the built-in

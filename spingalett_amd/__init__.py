@@ -96,12 +96,13 @@ PUBLIC_SYMBOLS = [
     "spingalett_set_dequant_mode", "spingalett_get_dequant_mode", "spingalett_forward_batch",
     "spingalett_forward_batch_device", "spingalett_hip_synchronize", "spingalett_hip_invalidate",
     "spingalett_hip_precision", "spingalett_hip_decode", "spingalett_hip_handle", "load_spingalett_memory",
+    "spingalett_evaluate_batch",
 ]
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
     "sphip_forward", "sphip_read_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
-    "sphip_layer_kernel_name",
+    "sphip_layer_kernel_name", "sphip_evaluate",
 ]
 
 
@@ -154,6 +155,9 @@ def lib():
     L.spingalett_forward_batch.restype = C.c_void_p
     L.spingalett_forward_batch_device.argtypes = [NetPtr, C.c_void_p, C.c_uint32, C.c_void_p]
     L.spingalett_forward_batch_device.restype = C.c_int
+    L.spingalett_evaluate_batch.argtypes = [NetPtr, C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(C.c_float),
+                                            C.c_void_p, C.POINTER(C.c_uint32)]
+    L.spingalett_evaluate_batch.restype = C.c_int
     L.spingalett_hip_synchronize.restype = C.c_int
     L.spingalett_hip_invalidate.argtypes = [NetPtr]; L.spingalett_hip_invalidate.restype = None
     L.spingalett_hip_precision.argtypes = [NetPtr]; L.spingalett_hip_precision.restype = C.c_int
@@ -246,6 +250,22 @@ def forward_batch(net, X):
         code, msg = last_error()
         raise SpingalettError(f"spingalett_forward_batch failed ({code}): {msg}")
     return out
+
+
+def evaluate_batch(net, X, T):
+    """spingalett_evaluate_batch: (total loss, predictions, number correct) of a labelled batch
+    (SIMD.c:522-552, Training.c:421-435)."""
+    nc = net.contents
+    X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, nc.topology[0])
+    T = np.ascontiguousarray(T, dtype=np.float32).reshape(X.shape[0], nc.topology[nc.layers - 1])
+    loss, correct = C.c_float(0), C.c_uint32(0)
+    pred = np.empty(X.shape[0], dtype=np.uint32)
+    rc = lib().spingalett_evaluate_batch(net, X.ctypes.data, T.ctypes.data, X.shape[0], C.byref(loss),
+                                         pred.ctypes.data, C.byref(correct))
+    if rc:
+        code, msg = last_error()
+        raise SpingalettError(f"spingalett_evaluate_batch failed ({code}): {msg}")
+    return loss.value, pred, correct.value
 
 
 def save_spingalett(net, filename: str, precision: int = PRECISION_FLOAT32, do_not_save_optimizer: bool = False):

@@ -144,6 +144,28 @@ int spingalett_forward_batch_device(NeuralNetwork *net, const float *d_inputs, u
     return 0;
 }
 
+int spingalett_evaluate_batch(NeuralNetwork *net, const float *inputs, const float *targets, uint32_t n,
+                              float *total_loss, uint32_t *predictions, uint32_t *correct)
+{
+    (void)sp_resolve_compute_mode();
+    sp_net *sn = checked(net, "evaluate_batch");
+    if (!sn) return 1;
+    if (!inputs || !targets || n == 0) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "evaluate_batch: null pointer or empty batch");
+        return 1;
+    }
+    if (net->loss_func >= LOSS_COUNT) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "evaluate_batch: unknown loss function");
+        return 1;
+    }
+    if (!ensure_device(sn)) return 1;
+    if (sphip_evaluate(sn->dev, inputs, targets, n, (int)net->loss_func, 0, total_loss, predictions, correct)) {
+        report(SPINGALETT_ERR_INVALID, "HIP back-end: evaluate_batch");
+        return 1;
+    }
+    return 0;
+}
+
 int spingalett_hip_synchronize(void)
 {
     if (sphip_synchronize()) {

@@ -1840,6 +1840,85 @@ __global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint
     g.C[idx] = apply_act(sum + bias, g.L.act);
 }
 
+// ---------------------------------------------------------------------------
+// evaluation of a batch of outputs (compute_sample_loss, SIMD.c:522-552;
+// batch_compute_loss, Training.c:421-435): one wave per sample
+// ---------------------------------------------------------------------------
+struct EvalArgs {
+    const float *y;        // [n][width] outputs
+    const float *target;   // [n][width]
+    float *loss;           // [n] per-sample loss
+    uint32_t *pred;        // [n] index of the first largest output
+    uint32_t *hit;         // [n] 1 when the target's first largest entry has the same index
+    uint32_t n, width;
+    int loss_func;         // 0 sum of squared differences, 1 cross-entropy
+    int sigmoid_out;       // cross-entropy in its binary form (output layer is a sigmoid)
+};
+
+__global__ __launch_bounds__(256) void sp_eval_rows(const EvalArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= a.n) return;
+    const float *o = a.y + (size_t)row * a.width, *tg = a.target + (size_t)row * a.width;
+    const float eps = 1e-9f;
+    float acc = 0.0f;
+    float bo = -__builtin_inff(), bt = -__builtin_inff();
+    uint32_t io = 0xFFFFFFFFu, it = 0xFFFFFFFFu;
+    for (uint32_t k = lane; k < a.width; k += kWave) {
+        const float ov = o[k], tv = tg[k];
+        if (a.loss_func == 0) {
+            const float d = ov - tv;
+            acc += d * d;
+        } else if (a.sigmoid_out) {
+            float c = ov < eps ? eps : ov;
+            c = c > 1.0f - eps ? 1.0f - eps : c;
+            acc -= tv * logf(c) + (1.0f - tv) * logf(1.0f - c);
+        } else {
+            const float c = ov < eps ? eps : ov;
+            acc -= tv * logf(c);
+        }
+        if (ov > bo || io == 0xFFFFFFFFu) { bo = ov; io = k; }
+        if (tv > bt || it == 0xFFFFFFFFu) { bt = tv; it = k; }
+    }
+    acc = wave_sum(acc);
+    // first largest element: larger value wins, equal values keep the lower index
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float vo = __shfl_xor(bo, s, kWave), vt = __shfl_xor(bt, s, kWave);
+        const uint32_t jo = __shfl_xor(io, s, kWave), jt = __shfl_xor(it, s, kWave);
+        if (jo != 0xFFFFFFFFu && (io == 0xFFFFFFFFu || vo > bo || (vo == bo && jo < io))) { bo = vo; io = jo; }
+        if (jt != 0xFFFFFFFFu && (it == 0xFFFFFFFFu || vt > bt || (vt == bt && jt < it))) { bt = vt; it = jt; }
+    }
+    if (lane == 0) {
+        a.loss[row] = acc;
+        a.pred[row] = io;
+        a.hit[row] = io == it ? 1u : 0u;
+    }
+}
+
+// one workgroup: total loss (added in FP64) and number of hits
+__global__ __launch_bounds__(1024) void sp_eval_total(const float *loss, const uint32_t *hit, uint32_t n, double *out_loss,
+                                                      uint32_t *out_hits)
+{
+    __shared__ double s_l[16];
+    __shared__ uint32_t s_h[16];
+    double l = 0.0;
+    uint32_t h = 0;
+    for (uint32_t i = threadIdx.x; i < n; i += 1024u) { l += (double)loss[i]; h += hit[i]; }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) { l += __shfl_xor(l, s, kWave); h += __shfl_xor(h, s, kWave); }
+    if ((threadIdx.x & 63) == 0) { s_l[threadIdx.x >> 6] = l; s_h[threadIdx.x >> 6] = h; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tl = 0.0;
+        uint32_t th = 0;
+        for (int w = 0; w < 16; ++w) { tl += s_l[w]; th += s_h[w]; }
+        *out_loss = tl;
+        *out_hits = th;
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -1879,6 +1958,8 @@ struct sphip_net {
     uint64_t total_neurons = 0;
     float *split_ws = nullptr;     // partial sums of the K splits of the thin-operand kernel
     uint64_t split_cap = 0;
+    float *eval_buf = nullptr;     // evaluation: outputs, staged targets, per-sample loss / prediction / hit, totals
+    uint64_t eval_cap = 0;
 };
 
 namespace {
@@ -2443,6 +2524,7 @@ void sphip_destroy(sphip_net *net)
     for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); }
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
     if (net->split_ws) (void)hipFree(net->split_ws);
+    if (net->eval_buf) (void)hipFree(net->eval_buf);
     for (int i = 0; i < 2; ++i) if (net->buf[i]) (void)hipFree(net->buf[i]);
     if (net->soft_tmp) (void)hipFree(net->soft_tmp);
     if (net->aq) (void)hipFree(net->aq);
@@ -2511,6 +2593,48 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
         HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
         HCHECK(hipStreamSynchronize(g_stream));
     }
+    return 0;
+}
+
+int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_t n, int loss_func, uint32_t flags,
+                   float *total_loss, uint32_t *predictions, uint32_t *correct)
+{
+    if (!net || !x || !targets || n == 0 || (loss_func != 0 && loss_func != 1))
+        return fail_msg("sphip_evaluate: invalid argument");
+    if (check_uploaded(net)) return 1;
+    if (reserve(net, n, false)) return 1;
+    const uint32_t width = net->topo[net->layers - 1];
+    const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * width;
+    const bool on_dev = (flags & SPHIP_X_ON_DEVICE) != 0;
+    // layout of the evaluation buffer (4-byte units): outputs | staged targets | loss | pred | hit | totals (16 bytes)
+    const uint64_t need = out_cnt * (on_dev ? 1u : 2u) + 3ull * n + 8u;
+    if (grow(&net->eval_buf, &net->eval_cap, need)) return 1;
+    float *d_y = net->eval_buf;
+    float *d_t = on_dev ? nullptr : net->eval_buf + out_cnt;
+    float *d_loss = net->eval_buf + out_cnt * (on_dev ? 1u : 2u);
+    uint32_t *d_pred = reinterpret_cast<uint32_t *>(d_loss + n);
+    uint32_t *d_hit = d_pred + n;
+    double *d_tot = reinterpret_cast<double *>((reinterpret_cast<uintptr_t>(d_hit + n) + 7u) & ~(uintptr_t)7u);
+    uint32_t *d_hits = reinterpret_cast<uint32_t *>(d_tot + 1);
+    const float *d_x = x;
+    if (!on_dev) {
+        if (grow(&net->stage_x, &net->stage_x_cap, in_cnt)) return 1;
+        HCHECK(hipMemcpyAsync(net->stage_x, x, in_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        HCHECK(hipMemcpyAsync(d_t, targets, out_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        d_x = net->stage_x;
+    }
+    if (enqueue_forward(net, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0)) return 1;
+    EvalArgs a{d_y, on_dev ? targets : d_t, d_loss, d_pred, d_hit, n, width, loss_func,
+               net->act[net->layers - 2] == A_SIGMOID ? 1 : 0};
+    sp_eval_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(a);
+    sp_eval_total<<<1, 1024, 0, g_stream>>>(d_loss, d_hit, n, d_tot, d_hits);
+    HCHECK(hipGetLastError());
+    struct { double loss; uint32_t hits; uint32_t pad; } tot;
+    HCHECK(hipMemcpyAsync(&tot, d_tot, 16, hipMemcpyDeviceToHost, g_stream));
+    if (predictions) HCHECK(hipMemcpyAsync(predictions, d_pred, (size_t)n * sizeof(uint32_t), hipMemcpyDeviceToHost, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    if (total_loss) *total_loss = (float)tot.loss;
+    if (correct) *correct = tot.hits;
     return 0;
 }
 

@@ -5,10 +5,10 @@ ALL_ACTS = ["sigmoid", "relu", "tanh", "leaky_relu", "foo52", "softmax", "none"]
 FORMATS = ["f32", "f16", "bf16", "i8", "i4", "i2"]
 
 
-def make_oracle_net(O, topology, acts, seed=0, init="he", bias_std=0.1):
+def make_oracle_net(O, topology, acts, seed=0, init="he", bias_std=0.1, loss=0):
     """A seeded FP32 net in the oracle's container. acts: names."""
     rng = np.random.default_rng(seed)
-    net = O.Net.new(topology, [O.ACT[a] for a in acts])
+    net = O.Net.new(topology, [O.ACT[a] for a in acts], loss)
     for l in range(len(topology) - 1):
         fan_in = topology[l]
         std = np.sqrt((2.0 if init == "he" else 1.0) / fan_in)

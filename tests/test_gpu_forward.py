@@ -336,3 +336,52 @@ def test_full_size_layer_unit_vector_probe(S):
         q = nib.astype(np.int32) - np.where(nib & 8, 16, 0)
         assert np.array_equal(gg[i], q.astype(F32)), k
     net.destroy()
+
+
+@pytest.mark.parametrize("fmt,acts,loss,n", [
+    ("i8", ["relu", "relu", "softmax"], 1, 300),         # classifier: cross-entropy on softmax outputs
+    ("bf16", ["tanh", "sigmoid"], 1, 77),                # sigmoid output layer: binary cross-entropy
+    ("i4", ["leaky_relu", "none"], 0, 3),                # squared error, vector path
+    ("f32", ["relu", "softmax"], 1, 1000),
+])
+def test_evaluate_batch_matches_oracle(S, O, fmt, acts, loss, n):
+    """spingalett_evaluate_batch = forward + compute_sample_loss (SIMD.c:522-552) summed over the
+    batch (Training.c:421-435) + per-sample argmax, all on the device.  The loss is compared with the
+    oracle's loss of the library's own outputs (so that only the evaluation step is under test), the
+    predictions with the argmax of those outputs."""
+    topo = [64, 128, 96, 10][:len(acts) + 1] if len(acts) == 3 else [48, 80, 12]
+    src = make_oracle_net(O, topo, acts, seed=71, loss=loss)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    assert net.contents.loss_func == loss
+    rng = np.random.default_rng(72)
+    X = rng.standard_normal((n, topo[0])).astype(F32)
+    labels = rng.integers(0, topo[-1], n)
+    T = np.eye(topo[-1], dtype=F32)[labels]
+    if loss == 0:
+        T = rng.standard_normal((n, topo[-1])).astype(F32)
+    Y = S.forward_batch(net, X)
+    total, pred, correct = S.evaluate_batch(net, X, T)
+    want = O.batch_loss(Y, T, loss, O.ACT[acts[-1]])
+    assert abs(total - want) <= 2e-5 * abs(want)
+    assert np.array_equal(pred, O.argmax_rows(Y))
+    assert correct == int((O.argmax_rows(Y) == O.argmax_rows(T)).sum())
+    # and end to end against the oracle's own forward, at the forward's tolerance
+    want_ref = O.batch_loss(ref.forward_batch(X), T, loss, O.ACT[acts[-1]])
+    assert abs(total - want_ref) <= (1e-3 if fmt == "f32" or n <= 4 else 3e-2) * abs(want_ref)
+    S.free_network(net)
+
+
+def test_evaluate_batch_argument_checks(S, O):
+    src = make_oracle_net(O, [16, 8], ["softmax"], seed=73, loss=1)
+    _, _, net = quantized_pair(O, S, src, "i8")
+    X = np.zeros((2, 16), F32)
+    T = np.zeros((2, 8), F32)
+    loss = C.c_float(0)
+    assert S.lib().spingalett_evaluate_batch(net, None, T.ctypes.data, 2, C.byref(loss), None, None) == 1
+    assert S.last_error()[0] == S.SPINGALETT_ERR_INVALID
+    S.clear_error()
+    assert S.lib().spingalett_evaluate_batch(net, X.ctypes.data, T.ctypes.data, 0, C.byref(loss), None, None) == 1
+    S.clear_error()
+    assert S.lib().spingalett_evaluate_batch(net, X.ctypes.data, T.ctypes.data, 2, C.byref(loss), None, None) == 0
+    assert loss.value == pytest.approx(0.0)                      # all-zero targets: nothing to add
+    S.free_network(net)

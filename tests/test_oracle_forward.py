@@ -107,3 +107,44 @@ def test_mid_size_against_numpy_matmul(O):
     if fn is not None:                                          # BLAS leg, when a BLAS is present
         sec, out = net.time_forward_batch(X, 1, fn, 2)
         assert np.max(np.abs(out - a)) / np.max(np.abs(a)) < 1e-5
+
+
+# ---------------------------------------------------------------------------
+# evaluation step (compute_sample_loss SIMD.c:522-552, batch_compute_loss Training.c:421-435)
+# ---------------------------------------------------------------------------
+def test_sample_loss_closed_forms(O):
+    """Pins: squared error of known vectors; cross-entropy of a one-hot target is -log of that
+    output; the 1e-9 clamp at zero; the binary form under a sigmoid output layer (symmetric in
+    (o, t) -> (1 - o, 1 - t)) with its clamp at one."""
+    SIG, SOFT, NONE = O.ACT["sigmoid"], O.ACT["softmax"], O.ACT["none"]
+    assert O.sample_loss([1.0, 2.0, -1.0], [0.5, 0.0, 1.0], 0, NONE) == pytest.approx(0.25 + 4.0 + 4.0, rel=1e-7)
+    o = np.array([0.2, 0.7, 0.1], np.float32)
+    assert O.sample_loss(o, [0, 1, 0], 1, SOFT) == pytest.approx(-np.log(0.7), rel=1e-6)
+    assert O.sample_loss(o, [0.5, 0.25, 0.25], 1, SOFT) == pytest.approx(
+        -(0.5 * np.log(0.2) + 0.25 * np.log(0.7) + 0.25 * np.log(0.1)), rel=1e-6)
+    # an output of exactly zero is clamped to 1e-9, not -inf
+    assert O.sample_loss([0.0, 1.0], [1, 0], 1, SOFT) == pytest.approx(-np.log(np.float32(1e-9)), rel=1e-6)
+    # sigmoid output layer: binary cross-entropy per output
+    a = O.sample_loss([0.3, 0.9], [1.0, 0.0], 1, SIG)
+    assert a == pytest.approx(-(np.log(0.3) + np.log(1 - 0.9)), rel=1e-5)
+    assert O.sample_loss([0.7, 0.1], [0.0, 1.0], 1, SIG) == pytest.approx(a, rel=1e-5)
+    # the upper clamp 1 - 1e-9 rounds to 1 in FP32, so an output of exactly 1 still reaches log(0):
+    # +inf against a target of 0, and 0 * -inf = NaN against a target of 1 (the arithmetic of
+    # SIMD.c:538-541 as written)
+    assert O.sample_loss([1.0], [0.0], 1, SIG) == float("inf")
+    assert np.isnan(O.sample_loss([1.0], [1.0], 1, SIG))
+    # a loss value outside the enum contributes nothing (neither branch runs)
+    assert O.sample_loss(o, [0, 1, 0], 2, SOFT) == 0.0
+
+
+def test_batch_loss_and_argmax(O):
+    rng = np.random.default_rng(3)
+    Y = rng.random((37, 11)).astype(np.float32)
+    Y /= Y.sum(1, keepdims=True)
+    T = np.eye(11, dtype=np.float32)[rng.integers(0, 11, 37)]
+    want = sum(-np.log(Y[i, T[i].argmax()].astype(np.float64)) for i in range(37))
+    assert O.batch_loss(Y, T, 1, O.ACT["softmax"]) == pytest.approx(want, rel=1e-5)
+    assert O.batch_loss(Y, T, 0, O.ACT["softmax"]) == pytest.approx(((Y.astype(np.float64) - T) ** 2).sum(), rel=1e-5)
+    assert np.array_equal(O.argmax_rows(Y), Y.argmax(1))
+    tie = np.array([[1.0, 3.0, 3.0, 2.0], [5.0, 5.0, 5.0, 5.0]], np.float32)
+    assert list(O.argmax_rows(tie)) == [1, 0]                      # first maximum
