@@ -39,7 +39,6 @@ typedef struct {
 /* flags of sphip_forward */
 #define SPHIP_X_ON_DEVICE   1u   /* x is a device pointer                       */
 #define SPHIP_Y_ON_DEVICE   2u   /* y is a device pointer (call does not wait)  */
-#define SPHIP_KEEP_LAYERS   4u   /* keep every layer's activations (n must be 1)*/
 #define SPHIP_FORCE_GEMM    8u   /* use the matrix-core path whatever n is      */
 #define SPHIP_FORCE_GEMV   16u   /* use the vector path (n <= 64)               */
 
@@ -79,9 +78,10 @@ SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *
  *   correct     : samples whose prediction equals the index of the target's first largest entry, or NULL */
 SPHIP_API int  sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_t n, int loss_func,
                               uint32_t flags, float *total_loss, uint32_t *predictions, uint32_t *correct);
-/* After a SPHIP_KEEP_LAYERS forward: copies all layers' activations to a host
- * array laid out like NeuralNetwork.neurons (Network.c:16-32). */
-SPHIP_API int  sphip_read_layers(sphip_net *net, float *host_neurons);
+/* forward_struct_arguments as its callers see it (Network.c:214-250): one sample, and every
+ * layer's activations (the input included) left in a host array laid out like
+ * NeuralNetwork.neurons (Network.c:16-32).  One call, one wait. */
+SPHIP_API int  sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons);
 
 /* The device form of the decoders in read_array_compressed
  * (Serialize.c:195-297) and fp16_to_float / bf16_to_float (:45-85): writes the

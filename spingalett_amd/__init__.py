@@ -31,7 +31,7 @@ SPINGALETT_OK, SPINGALETT_ERR_ALLOC, SPINGALETT_ERR_INVALID = 0, 1, 2
 DEQUANT_STRICT, DEQUANT_RELEASE = 0, 1
 LOG_DEBUG, LOG_INFO, LOG_WARNING, LOG_ERROR, LOG_NONE = range(5)
 
-SPHIP_X_ON_DEVICE, SPHIP_Y_ON_DEVICE, SPHIP_KEEP_LAYERS, SPHIP_FORCE_GEMM, SPHIP_FORCE_GEMV = 1, 2, 4, 8, 16
+SPHIP_X_ON_DEVICE, SPHIP_Y_ON_DEVICE, SPHIP_FORCE_GEMM, SPHIP_FORCE_GEMV = 1, 2, 8, 16
 
 
 class NeuralNetwork(C.Structure):
@@ -100,7 +100,7 @@ PUBLIC_SYMBOLS = [
 ]
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
-    "sphip_forward", "sphip_read_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
+    "sphip_forward", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
     "sphip_layer_kernel_name", "sphip_evaluate",
 ]
@@ -173,7 +173,7 @@ def lib():
     L.sphip_upload_array.restype = C.c_int
     L.sphip_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32]
     L.sphip_forward.restype = C.c_int
-    L.sphip_read_layers.argtypes = [C.c_void_p, C.c_void_p]; L.sphip_read_layers.restype = C.c_int
+    L.sphip_forward_layers.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]; L.sphip_forward_layers.restype = C.c_int
     L.sphip_decode.argtypes = [C.c_void_p, C.c_uint32, C.c_int, C.c_int, C.c_void_p]; L.sphip_decode.restype = C.c_int
     L.sphip_synchronize.restype = C.c_int
     L.sphip_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]; L.sphip_malloc.restype = C.c_int

@@ -106,7 +106,7 @@ float *sp_hip_forward_single(sp_net *sn, const float *input)
     NeuralNetwork *net = &sn->pub;
     if (!ensure_device(sn)) return NULL;
     float *out = net->neurons + net->neuron_offsets[net->layers - 1];
-    if (sphip_forward(sn->dev, input, 1, out, SPHIP_KEEP_LAYERS) || sphip_read_layers(sn->dev, net->neurons)) {
+    if (sphip_forward_layers(sn->dev, input, net->neurons)) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: forward");
         return NULL;
     }

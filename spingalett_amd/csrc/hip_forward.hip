@@ -1841,6 +1841,31 @@ __global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint
 }
 
 // ---------------------------------------------------------------------------
+// small copies (host staging of single-sample forwards)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sp_copy32(const float *__restrict__ src, float *__restrict__ dst, uint64_t n)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+// gathers up to 16 layer slots (16-byte aligned starts) into the dense neurons layout
+struct PackArgs {
+    const float *src;
+    float *dst;
+    uint32_t count;
+    uint32_t src_off[16], dst_off[16], len[16];
+};
+
+__global__ __launch_bounds__(256) void sp_pack_layers(const PackArgs a)
+{
+    const uint32_t s = blockIdx.y;
+    if (s >= a.count) return;
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < a.len[s]; i += gridDim.x * 256u)
+        a.dst[a.dst_off[s] + i] = a.src[a.src_off[s] + i];
+}
+
+// ---------------------------------------------------------------------------
 // evaluation of a batch of outputs (compute_sample_loss, SIMD.c:522-552;
 // batch_compute_loss, Training.c:421-435): one wave per sample
 // ---------------------------------------------------------------------------
@@ -1950,7 +1975,11 @@ struct sphip_net {
     uint32_t aq_cap_n = 0;
     float *soft_tmp = nullptr;     // FP32 logits of a softmax layer
     uint64_t soft_cap = 0;
-    float *layers_buf = nullptr;   // per-layer activations of a KEEP_LAYERS forward
+    float *layers_buf = nullptr;   // all activations of a single-sample forward, each layer at a 16-byte aligned slot
+    std::vector<uint32_t> slot_off;  // start of each layer's slot (floats)
+    uint64_t slots_total = 0;
+    float *pin_in = nullptr, *pin_out = nullptr;   // pinned host staging of small inputs / outputs
+    uint64_t pin_in_cap = 0, pin_out_cap = 0;
     float *stage_x = nullptr;      // device staging of host inputs / outputs
     float *stage_y = nullptr;
     uint64_t stage_x_cap = 0, stage_y_cap = 0;
@@ -2342,7 +2371,7 @@ int reserve(sphip_net *net, uint32_t n, bool keep_layers)
         net->aq_valid_layer = 0;
     }
     if (keep_layers && !net->layers_buf)
-        HCHECK(hipMalloc((void **)&net->layers_buf, net->total_neurons * sizeof(float)));
+        HCHECK(hipMalloc((void **)&net->layers_buf, net->slots_total * sizeof(float)));
     if (net->prec == F32 && n > 64) {
         uint64_t ws = 0;
         for (uint32_t l = 1; l < net->layers; ++l) {
@@ -2409,9 +2438,10 @@ int check_uploaded(const sphip_net *net)
 
 // Enqueues every kernel of one forward.  d_x, d_y are device pointers.
 // only_layer != 0 restricts the launch to the main kernel of that layer.
-int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags, uint32_t only_layer)
+// keep (n == 1): every layer's output goes to its slot of layers_buf, d_x must be slot 0 and d_y the last slot.
+int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags, uint32_t only_layer,
+                    bool keep = false)
 {
-    const bool keep = (flags & SPHIP_KEEP_LAYERS) != 0;
     const Regime reg = pick_regime(net, n, flags);
     const bool f16t = net->prec != BF16;          // 16-bit activation type of the matrix-core path
     const uint32_t last = net->layers - 1;
@@ -2426,15 +2456,12 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
     } else if (reg == R_GEMM16) {
         in = net->buf[1];
     }
-    if (keep)
-        HCHECK(hipMemcpyAsync(net->layers_buf, d_x, (size_t)net->topo[0] * sizeof(float), hipMemcpyDeviceToDevice, g_stream));
 
-    uint64_t noff = net->topo[0];
     for (uint32_t l = 1; l <= last; ++l) {
         const LayerArgs L = make_layer_args(net, l);
         const bool softmax = net->act[l - 1] == A_SOFTMAX;
         const bool is_last = l == last;
-        void *dst = is_last ? (void *)d_y : net->buf[(l + 1) & 1];
+        void *dst = is_last ? (void *)d_y : keep ? (void *)(net->layers_buf + net->slot_off[l]) : net->buf[(l + 1) & 1];
         // logits of a softmax layer go to FP32 scratch first
         void *main_out = softmax ? (void *)net->soft_tmp : dst;
         const int out_f32 = (reg != R_GEMM16) || is_last || softmax;
@@ -2457,11 +2484,7 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
             const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
             sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(net->soft_tmp, dst, kind, n, net->topo[l]);
         }
-        if (keep)     // n == 1 and FP32 activations: mirror the layer into the neurons-shaped buffer
-            HCHECK(hipMemcpyAsync(net->layers_buf + noff, dst, (size_t)net->topo[l] * sizeof(float),
-                                  hipMemcpyDeviceToDevice, g_stream));
         in = dst;
-        noff += net->topo[l];
     }
     HCHECK(hipGetLastError());
     return 0;
@@ -2500,6 +2523,8 @@ int sphip_create(const sphip_desc *desc, sphip_net **out)
     for (uint32_t l = 0; l < desc->layers; ++l) {
         if (net->topo[l] > net->max_width) net->max_width = net->topo[l];
         net->total_neurons += net->topo[l];
+        net->slot_off.push_back((uint32_t)net->slots_total);
+        net->slots_total += ((uint64_t)net->topo[l] + 3u) & ~3ull;
     }
     for (uint32_t l = 0; l + 1 < desc->layers; ++l) {
         DevArray &w = net->W[l], &b = net->B[l];
@@ -2531,6 +2556,8 @@ void sphip_destroy(sphip_net *net)
     if (net->aq_inv) (void)hipFree(net->aq_inv);
     if (net->aq_dsum) (void)hipFree(net->aq_dsum);
     if (net->layers_buf) (void)hipFree(net->layers_buf);
+    if (net->pin_in) (void)hipHostFree(net->pin_in);
+    if (net->pin_out) (void)hipHostFree(net->pin_out);
     if (net->stage_x) (void)hipFree(net->stage_x);
     if (net->stage_y) (void)hipFree(net->stage_y);
     delete net;
@@ -2570,29 +2597,93 @@ int sphip_clone(const sphip_net *src, sphip_net **out)
     return 0;
 }
 
+// Small host inputs travel through a pinned staging buffer and a copy kernel; small outputs are
+// written by the last layer's kernel straight into pinned memory (scattered stores over PCIe do
+// not pay beyond a few thousand values), and the call ends with one stream synchronisation.
+static const uint64_t kSmallIn = 256u * 1024u, kSmallOut = 4096u;
+
+static int grow_pinned(float **p, uint64_t *cap, uint64_t need)
+{
+    if (need <= *cap) return 0;
+    if (*p) { HCHECK(hipHostFree(*p)); *p = nullptr; }
+    *cap = 0;
+    HCHECK(hipHostMalloc((void **)p, need * sizeof(float), hipHostMallocDefault));
+    *cap = need;
+    return 0;
+}
+
 int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t flags)
 {
     if (!net || !x || !y || n == 0) return fail_msg("sphip_forward: invalid argument");
-    if ((flags & SPHIP_KEEP_LAYERS) && n != 1) return fail_msg("sphip_forward: SPHIP_KEEP_LAYERS needs n == 1");
     if (check_uploaded(net)) return 1;
-    if (reserve(net, n, (flags & SPHIP_KEEP_LAYERS) != 0)) return 1;
+    if (reserve(net, n, false)) return 1;
     const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * net->topo[net->layers - 1];
     const float *d_x = x;
     float *d_y = y;
+    bool y_pinned = false;
     if (!(flags & SPHIP_X_ON_DEVICE)) {
         if (grow(&net->stage_x, &net->stage_x_cap, in_cnt)) return 1;
-        HCHECK(hipMemcpyAsync(net->stage_x, x, in_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        if (in_cnt <= kSmallIn) {
+            if (grow_pinned(&net->pin_in, &net->pin_in_cap, in_cnt)) return 1;
+            memcpy(net->pin_in, x, in_cnt * sizeof(float));
+            sp_copy32<<<(uint32_t)((in_cnt + 255) / 256), 256, 0, g_stream>>>(net->pin_in, net->stage_x, in_cnt);
+        } else {
+            HCHECK(hipMemcpyAsync(net->stage_x, x, in_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        }
         d_x = net->stage_x;
     }
     if (!(flags & SPHIP_Y_ON_DEVICE)) {
-        if (grow(&net->stage_y, &net->stage_y_cap, out_cnt)) return 1;
-        d_y = net->stage_y;
+        if (out_cnt <= kSmallOut) {
+            if (grow_pinned(&net->pin_out, &net->pin_out_cap, out_cnt)) return 1;
+            d_y = net->pin_out;
+            y_pinned = true;
+        } else {
+            if (grow(&net->stage_y, &net->stage_y_cap, out_cnt)) return 1;
+            d_y = net->stage_y;
+        }
     }
     if (enqueue_forward(net, d_x, n, d_y, flags, 0)) return 1;
     if (!(flags & SPHIP_Y_ON_DEVICE)) {
-        HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
+        if (!y_pinned) HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
         HCHECK(hipStreamSynchronize(g_stream));
+        if (y_pinned) memcpy(y, net->pin_out, out_cnt * sizeof(float));
     }
+    return 0;
+}
+
+int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
+{
+    if (!net || !x || !host_neurons) return fail_msg("sphip_forward_layers: invalid argument");
+    if (check_uploaded(net)) return 1;
+    if (reserve(net, 1, true)) return 1;
+    const uint32_t last = net->layers - 1;
+    if (grow_pinned(&net->pin_in, &net->pin_in_cap, net->topo[0])) return 1;
+    if (grow_pinned(&net->pin_out, &net->pin_out_cap, net->total_neurons)) return 1;
+    memcpy(net->pin_in, x, (size_t)net->topo[0] * sizeof(float));
+    sp_copy32<<<(net->topo[0] + 255) / 256, 256, 0, g_stream>>>(net->pin_in, net->layers_buf, net->topo[0]);
+    if (enqueue_forward(net, net->layers_buf, 1, net->layers_buf + net->slot_off[last], 0, 0, true)) return 1;
+    // all slots, densely packed, straight into pinned memory
+    uint32_t dense = 0;
+    for (uint32_t l0 = 0; l0 < net->layers; l0 += 16) {
+        PackArgs pa{};
+        pa.src = net->layers_buf;
+        pa.dst = net->pin_out;
+        pa.count = net->layers - l0 < 16 ? net->layers - l0 : 16;
+        uint32_t widest = 1;
+        for (uint32_t i = 0; i < pa.count; ++i) {
+            pa.src_off[i] = net->slot_off[l0 + i];
+            pa.dst_off[i] = dense;
+            pa.len[i] = net->topo[l0 + i];
+            dense += net->topo[l0 + i];
+            if (pa.len[i] > widest) widest = pa.len[i];
+        }
+        uint32_t gx = (widest + 255) / 256;
+        if (gx > 64) gx = 64;
+        sp_pack_layers<<<dim3(gx, pa.count), 256, 0, g_stream>>>(pa);
+    }
+    HCHECK(hipGetLastError());
+    HCHECK(hipStreamSynchronize(g_stream));
+    memcpy(host_neurons, net->pin_out, net->total_neurons * sizeof(float));
     return 0;
 }
 
@@ -2635,14 +2726,6 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
     HCHECK(hipStreamSynchronize(g_stream));
     if (total_loss) *total_loss = (float)tot.loss;
     if (correct) *correct = tot.hits;
-    return 0;
-}
-
-int sphip_read_layers(sphip_net *net, float *host_neurons)
-{
-    if (!net || !host_neurons || !net->layers_buf) return fail_msg("sphip_read_layers: no kept activations");
-    HCHECK(hipMemcpyAsync(host_neurons, net->layers_buf, net->total_neurons * sizeof(float), hipMemcpyDeviceToHost, g_stream));
-    HCHECK(hipStreamSynchronize(g_stream));
     return 0;
 }
 
@@ -2751,7 +2834,7 @@ int sphip_time_forward(sphip_net *const *nets, int count, const float *d_x, uint
                        uint32_t flags, int iters, float *ms)
 {
     if (!d_x || !d_y || n == 0) return fail_msg("sphip_time_forward: invalid argument");
-    return time_common(nets, count, d_x, n, d_y, flags & ~SPHIP_KEEP_LAYERS, iters, ms, 0);
+    return time_common(nets, count, d_x, n, d_y, flags, iters, ms, 0);
 }
 
 int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t n, uint32_t flags,
@@ -2765,7 +2848,7 @@ int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t
         if (grow(&nets[i]->stage_y, &nets[i]->stage_y_cap, (uint64_t)n * nets[i]->topo[nets[i]->layers - 1])) return 1;
         if (grow(&nets[i]->stage_x, &nets[i]->stage_x_cap, (uint64_t)n * nets[i]->topo[0])) return 1;
     }
-    return time_common(nets, count, nets[0]->stage_x, n, nets[0]->stage_y, flags & ~SPHIP_KEEP_LAYERS, iters, ms, layer);
+    return time_common(nets, count, nets[0]->stage_x, n, nets[0]->stage_y, flags, iters, ms, layer);
 }
 
 const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, uint32_t flags)
