@@ -1122,6 +1122,16 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 template <int OFF>
 __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
 
@@ -1248,25 +1258,27 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)As + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
     const uint32_t lds_w = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)Ws + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
     const bool loader = wave_s < HALF;
-    // part = -1: the whole tile; 0, 1, 2: the share issued in front of k-step `part` of the running stage
-    auto issue_direct = [&](int buf, uint32_t k0, int part) {
+    // the idx-th load instruction of a loader wave's tile (A first, then W); idx is a constant once
+    // the caller's loops are unrolled
+    constexpr int DMA_TOTAL = A_DUTY + (W_DIRECT ? W_DUTY : 0);
+    auto issue_one = [&](int buf, uint32_t k0, int idx) {
         if (!loader) return;
-        const char *ab = a_base + (size_t)k0 * 2u, *wb = w_base + (size_t)k0 * 2u;
-        constexpr int TOTAL = A_DUTY + (W_DIRECT ? W_DUTY : 0);
 #pragma unroll
-        for (int d = 0; d < A_DUTY; ++d) {
-            const int slot = d * 3 / TOTAL;
-            if (part < 0 || part == slot)
-                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), a_voff[d], ab);
-        }
+        for (int d = 0; d < A_DUTY; ++d)
+            if (d == idx)
+                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), a_voff[d],
+                          a_base + (size_t)k0 * 2u);
         if constexpr (W_DIRECT) {
 #pragma unroll
-            for (int d = 0; d < W_DUTY; ++d) {
-                const int slot = (A_DUTY + d) * 3 / TOTAL;
-                if (part < 0 || part == slot)
-                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), w_voff[d], wb);
-            }
+            for (int d = 0; d < W_DUTY; ++d)
+                if (A_DUTY + d == idx)
+                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), w_voff[d],
+                              w_base + (size_t)k0 * 2u);
         }
+    };
+    auto issue_direct = [&](int buf, uint32_t k0) {            // the whole tile at once (prologue)
+#pragma unroll
+        for (int idx = 0; idx < DMA_TOTAL; ++idx) issue_one(buf, k0, idx);
     };
     auto load_w_regs = [&](uint32_t k0) {
         if constexpr (!W_DIRECT) {
@@ -1319,6 +1331,9 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     }
     u32x4 fa[2][TM], fb[2][TN];
 
+    // A loader wave slips one load instruction behind each of the first MFMAs of k-steps 0..2: the
+    // matrix pipe is busy for eight passes after every issue, and the address unit takes the load meanwhile.
+    constexpr int DPS = (DMA_TOTAL + 2) / 3;              // load instructions per k-step
     auto stage = [&](auto cur_c, bool more, uint32_t knext) {
         constexpr int CUR = decltype(cur_c)::value;
         if (more) load_w_regs(knext);
@@ -1330,7 +1345,6 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             if (ks < 3) {
                 frag_reads<CUR * BM * BK * 2, TM>(fa[cs ^ 1], va[ks + 1]);
                 frag_reads<CUR * BN * BK * 2, TN>(fb[cs ^ 1], vw[ks + 1]);
-                if (more) issue_direct(CUR ^ 1, knext, ks);
                 asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
             } else {
                 asm volatile("s_waitcnt lgkmcnt(0)");
@@ -1355,6 +1369,11 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
                         __builtin_memcpy(&b, &fb[cs][j], 16);
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
                     }
+                    if (more && ks < 3 && i * TN + j < DPS) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(CUR ^ 1, knext, ks * DPS + i * TN + j);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -1367,7 +1386,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     const uint32_t kbeg = g.kper ? blockIdx.y * g.kper : 0u;
     const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
     const uint32_t ktiles = (kend - kbeg) / BK;
-    issue_direct(0, kbeg, -1);
+    issue_direct(0, kbeg);
     load_w_regs(kbeg);
     store_w_regs(0);
     asm volatile("s_waitcnt vmcnt(0)");
