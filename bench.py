@@ -50,7 +50,7 @@ WORKLOADS = {
     "C4": dict(topo=[8192] * 9 + [1000], acts=["leaky", "foo52"] * 4 + ["softmax"], init=["he"] * 9,
                prec=S.PRECISION_BFLOAT16, inputs="n01", batches=[8192]),
     "C5": dict(topo=[2048, 8192, 8192, 8192, 8192, 1000], acts=["sigmoid", "relu", "relu", "tanh", "softmax"],
-               init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1, 64, 4096, 65536]),
+               init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1, 8, 64, 512, 4096, 65536]),
 }
 
 
@@ -58,7 +58,7 @@ def compute_dtype(prec: int, n: int) -> str:
     """Arithmetic type of the path taken (not a precision claim about the weights)."""
     if prec == S.PRECISION_FLOAT32:
         return "f32"
-    if n <= 64:
+    if n <= 4:
         return "i8 (exact integer digits, f32 accumulate)" if prec >= S.PRECISION_INT8 else "f32"
     return "bf16" if prec == S.PRECISION_BFLOAT16 else "f16"
 
@@ -164,10 +164,12 @@ def time_workload(copies, topo, n, x_host, steps, warmup):
 
 # HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (summaries and calibration factors: profiles/sp_gemm16_big_C4_bf16_b8192.md,
-# profiles/sp_gemv_i8mfma_C3_int4_b1.md).  Keyed by (kernel, [n, N, K]); None when not profiled.
+# profiles/sp_gemv_i8mfma_C3_int4_b1.md, profiles/sp_skinny16_C3_int4_b64.md).
+# Keyed by (kernel, [n, N, K]); None when not profiled.
 PROFILED_TRAFFIC = {
-    ("sp_gemm16_big", (8192, 8192, 8192)): (791942 * 2.0 + 187433 * 1.0) * 1024,
-    ("sp_gemv_i8mfma", (1, 16384, 16384)): (66051 * 2.0 + 64 * 1.0) * 1024,
+    ("sp_gemm16_big", (8192, 8192, 8192)): (790488 * 2.0 + 186515 * 1.0) * 1024,
+    ("sp_gemv_i8mfma", (1, 16384, 16384)): (68204 * 2.0 + 64 * 1.0) * 1024,
+    ("sp_skinny16", (64, 16384, 16384)): ((74139 + 8221) * 2.0 + (16384 + 2048) * 1.0) * 1024,
 }
 
 
@@ -236,6 +238,15 @@ def run_workload(name, batches, steps, warmup, want_output=False):
                    mfma_frac=fl / (ms_ev * 1e-3) / (FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK),
                    copies=len(copies), finite=bool(np.isfinite(y).all()))
         row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
+        if n == 1:
+            # the public forward(): host pointer in, all activations mirrored into net->neurons (PCIe both ways)
+            x1 = np.ascontiguousarray(x[0])
+            for _ in range(20):
+                S.forward(net, x1)
+            t1 = time.perf_counter()
+            for _ in range(200):
+                S.forward(net, x1)
+            row["public_forward_us"] = (time.perf_counter() - t1) / 200 * 1e6
         rows.append(row)
     return dict(net=net, path=path, copies=copies, clones=clones, rows=rows, build_s=build_s)
 
