@@ -933,12 +933,65 @@ __device__ __forceinline__ uint32_t int_to_t16(int q)
     }
 }
 
-// unpack one 32-bit word of codes into 16-bit floats, written as packed pairs
+// packed FP16 subtraction a - c (two lanes at once)
+__device__ __forceinline__ uint32_t h2_sub(uint32_t v, uint32_t c)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 a, b;
+    __builtin_memcpy(&a, &v, 4);
+    __builtin_memcpy(&b, &c, 4);
+    a = a - b;
+    uint32_t r;
+    __builtin_memcpy(&r, &a, 4);
+    return r;
+}
+
+// unpack one 32-bit word of codes into 16-bit floats, written as packed pairs (codes 0 1, 2 3, ...)
 template <int FMT, bool F16T>
 __device__ __forceinline__ void unpack_word16(uint32_t w, uint32_t *o)
 {
     constexpr int bits = fmt_bits(FMT);
     constexpr int cnt = 32 / bits;
+    if constexpr (F16T && (FMT == I8 || FMT == I4 || FMT == I2)) {
+        // A field masked in place and XORed onto an FP16 constant whose last mantissa bit weighs as much as
+        // the field's lowest bit (the same XOR flips the sign bit: two's complement -> offset binary) reads
+        // as constant + offset + code; one packed subtraction leaves the codes of two fields, exactly.  The
+        // pairs come out as (code k, code k + cnt/2) and a byte permute puts neighbours together.
+        constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;      // low / high halves of two words
+        if constexpr (FMT == I8) {
+            const uint32_t t0 = h2_sub((w & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);            // codes 0, 2
+            const uint32_t t1 = h2_sub(((w >> 8) & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);     // codes 1, 3
+            o[0] = __builtin_amdgcn_perm(t1, t0, LO);
+            o[1] = __builtin_amdgcn_perm(t1, t0, HI);
+        } else if constexpr (FMT == I4) {
+            const uint32_t y = w >> 8;
+            const uint32_t t0 = h2_sub((w & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);            // codes 0, 4
+            const uint32_t t1 = h2_sub((w & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);            // codes 1, 5
+            const uint32_t t2 = h2_sub((y & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);            // codes 2, 6
+            const uint32_t t3 = h2_sub((y & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);            // codes 3, 7
+            o[0] = __builtin_amdgcn_perm(t1, t0, LO);
+            o[1] = __builtin_amdgcn_perm(t3, t2, LO);
+            o[2] = __builtin_amdgcn_perm(t1, t0, HI);
+            o[3] = __builtin_amdgcn_perm(t3, t2, HI);
+        } else {
+            const uint32_t y = w >> 10;
+            uint32_t p[8];                                                                        // codes k, k + 8
+            p[0] = h2_sub((w & 0x00030003u) ^ 0x64026402u, 0x64026402u);
+            p[1] = h2_sub((w & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);
+            p[2] = h2_sub((w & 0x00300030u) ^ 0x54205420u, 0x54205420u);
+            p[3] = h2_sub((w & 0x00C000C0u) ^ 0x4C804C80u, 0x4C804C80u);
+            p[4] = h2_sub((w & 0x03000300u) ^ 0x46004600u, 0x46004600u);
+            p[5] = h2_sub((y & 0x00030003u) ^ 0x64026402u, 0x64026402u);
+            p[6] = h2_sub((y & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);
+            p[7] = h2_sub((y & 0x00300030u) ^ 0x54205420u, 0x54205420u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                o[q]     = __builtin_amdgcn_perm(p[2 * q + 1], p[2 * q], LO);
+                o[4 + q] = __builtin_amdgcn_perm(p[2 * q + 1], p[2 * q], HI);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < cnt; j += 2) {
         int q0 = (int)(w << (32 - bits - bits * j)) >> (32 - bits);
