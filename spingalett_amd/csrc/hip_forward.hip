@@ -17,6 +17,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -81,8 +82,12 @@ int g_gemv_waves = 0;       // 0: automatic
 int g_gemv_lds_kib = 64;
 int g_gemm_variant = 1;     // 0: 128x128 tiles only (tuning switch)
 
+std::mutex g_init_mutex;
+
+// One stream per process (default priority), created at first use; safe to call from several threads.
 int ensure_stream()
 {
+    std::lock_guard<std::mutex> lock(g_init_mutex);
     if (g_stream) return 0;
     int cnt = 0;
     HCHECK(hipGetDeviceCount(&cnt));

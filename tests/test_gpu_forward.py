@@ -385,3 +385,57 @@ def test_evaluate_batch_argument_checks(S, O):
     assert S.lib().spingalett_evaluate_batch(net, X.ctypes.data, T.ctypes.data, 2, C.byref(loss), None, None) == 0
     assert loss.value == pytest.approx(0.0)                      # all-zero targets: nothing to add
     S.free_network(net)
+
+
+def test_full_size_gemm_layer_properties(S):
+    """8192 x 8192 BF16 at batch 8192 (one layer of config 4, the tiled GEMM at its benchmark shape):
+    one-hot rows read columns of W exactly, duplicated rows give identical outputs wherever they sit
+    in the batch, and random rows agree with FP64 dot products of the BF16-rounded operands."""
+    K = N = n = 8192
+    rng = np.random.default_rng(81)
+    w = (rng.standard_normal(N * K, dtype=F32) * F32(0.02))
+    codes = (w.view(np.uint32) >> 16).astype(np.uint16)
+    net = S.DeviceNet([K, N], [S.ACT_NONE], S.PRECISION_BFLOAT16)
+    net.upload(0, 0, codes)
+    net.upload(0, 1, np.zeros(N, np.uint16))
+    Wd = (codes.astype(np.uint32) << 16).view(F32).reshape(N, K)
+    X = rng.standard_normal((n, K), dtype=F32)
+    hot = [0, 1, 255, 256, 4097, 8191]
+    for i, r in enumerate(hot):
+        X[r] = 0
+        X[r, (r * 37 + 5) % K] = 1.0
+    X[7000] = X[3]                                                   # duplicates in different tiles
+    X[8190] = X[3]
+    Y = net.forward(X)
+    for r in hot:
+        assert np.array_equal(Y[r], Wd[:, (r * 37 + 5) % K]), r
+    assert np.array_equal(Y[7000], Y[3]) and np.array_equal(Y[8190], Y[3])
+    for r in (3, 1234, 8189):
+        xb = ((X[r].view(np.uint32) + 0x7FFF + ((X[r].view(np.uint32) >> 16) & 1)) & 0xFFFF0000).view(F32)   # BF16 RNE
+        want = Wd.astype(np.float64) @ xb.astype(np.float64)
+        assert rel_max_abs(Y[r], want) <= 1e-4, r                    # products exact, FP32 accumulation over 8192 terms
+    net.destroy()
+
+
+def test_full_batch_int2_first_layer_properties(S):
+    """2048 -> 8192 INT2 at batch 65536 (first layer of config 5 at the top of its sweep): every row of the
+    batch is one of 97 distinct inputs; equal inputs must give bit-identical outputs in all 65536 positions,
+    and the distinct ones agree with FP64 on the decoded codes."""
+    K, N, n = 2048, 8192, 65536
+    rng = np.random.default_rng(82)
+    net = S.DeviceNet([K, N], [S.ACT_TANH], S.PRECISION_INT2)
+    net.upload(0, 0, rng.integers(0, 256, size=N * K // 4, dtype=np.uint8), 0.03)
+    net.upload(0, 1, rng.integers(0, 256, size=N // 4, dtype=np.uint8), 0.2)
+    W = net.decode(0, 0).astype(np.float64).reshape(N, K)
+    b = net.decode(0, 1).astype(np.float64)
+    base = (rng.random((97, K), dtype=F32) * 2 - 1)
+    idx = rng.integers(0, 97, n)
+    Y = net.forward(base[idx])
+    first = {int(v): int(np.nonzero(idx == v)[0][0]) for v in range(97)}
+    ref_rows = np.stack([Y[first[int(v)]] for v in idx[::997]])
+    assert np.array_equal(Y[::997], ref_rows)
+    assert np.array_equal(Y[np.nonzero(idx == 5)[0]], np.broadcast_to(Y[first[5]], (int((idx == 5).sum()), N)))
+    want = np.tanh(base[:8].astype(np.float16).astype(np.float64) @ W.T + b)
+    got = np.stack([Y[first[v]] for v in range(8)])
+    assert rel_max_abs(got, want) <= 2e-3
+    net.destroy()
