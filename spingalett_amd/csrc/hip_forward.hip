@@ -1619,6 +1619,14 @@ __device__ __forceinline__ void skinny_emit(const SkinnyArgs &a, uint32_t c, uin
     else reinterpret_cast<uint16_t *>(a.C)[o] = f32_to_t16<F16T>(v);
 }
 
+// 16 bytes per lane from scalar base + 32-bit lane offset + immediate.  Inline assembly: the compiler's
+// wait-count bookkeeping does not see the load, the caller waits with s_waitcnt vmcnt before using dst.
+template <int OFF>
+__device__ __forceinline__ void load16_async(u32x4 &dst, uint32_t voff, const void *sbase)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+}
+
 template <int FMT, bool F16T, int RT, int CT>
 __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
 {
@@ -1639,11 +1647,23 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
     const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
     const size_t row_bytes = (size_t)K * F::bits / 8u;
 
-    const uint8_t *srow[RT];
+    // per-lane byte offsets (32-bit: the host checks that both operands span less than 4 GiB)
+    uint32_t svoff[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const uint32_t r = row0 + rt * 32u + n31;
-        srow[rt] = a.stream + (size_t)(r < a.R ? r : a.R - 1) * row_bytes;
+        svoff[rt] = (uint32_t)((size_t)(r < a.R ? r : a.R - 1) * row_bytes) + h * 16u;
+    }
+    uint32_t tvoff[UPT][2];
+    bool trow_ok[UPT];
+#pragma unroll
+    for (int q = 0; q < UPT; ++q) {
+        const uint32_t u = (uint32_t)t + 256u * q;
+        const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
+        const uint32_t c = cbase + row;
+        trow_ok[q] = u < (uint32_t)UNITS && c < a.NC;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) tvoff[q][e] = trow_ok[q] ? (uint32_t)(((size_t)c * K + uc * 16u + 8u * e) * 2u) : 0u;
     }
 
     f32x16 acc[RT][CT];
@@ -1654,53 +1674,85 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[rt][ct][r] = 0.0f;
 
-    auto load_stream = [&](uint32_t kc0, uint4 (&dst)[RT][LPC]) {
+    // Loads are issued two chunks ahead for the streamed rows and one ahead for the thin block.  A chunk past
+    // the end is clamped to the last one (a redundant load) so that the number of loads in flight is always the
+    // same.  In the last chunk a lane load that would start past the end of its row reads the row's start
+    // instead; what it fetched is masked (16-bit values) or meets zeros of the thin operand (integer codes).
+    constexpr int S_LOADS = RT * LPC, T_LOADS = UPT * 2;
+    const uint32_t last_chunk = nchunks - 1;
+    auto issue_stream = [&](uint32_t ch, u32x4 (&dst)[RT][LPC]) {
+        if (ch < last_chunk) {
+            const uint8_t *sb = a.stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
 #pragma unroll
-        for (int i = 0; i < LPC; ++i) {
-            const uint32_t k = kc0 + (2u * i + h) * EPL;            // first code of this lane load
-            const bool valid = k < K;                                // rows are whole numbers of lane loads
-            const size_t off = (size_t)(valid ? k : 0u) * F::bits / 8u;
-            // integer codes past the end of a row meet zeros of the thin operand; 16-bit values there
-            // could be NaN or infinite and are masked
-            const uint32_t keep = (F::bits == 16 && !valid) ? 0u : 0xFFFFFFFFu;
+            for (int i = 0; i < LPC; ++i)
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                uint4 v = *reinterpret_cast<const uint4 *>(srow[rt] + off);
-                if constexpr (F::bits == 16) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
-                dst[rt][i] = v;
+                for (int rt = 0; rt < RT; ++rt) {
+                    if (i == 0) load16_async<0>(dst[rt][i], svoff[rt], sb);
+                    else if (i == 1) load16_async<32>(dst[rt][i], svoff[rt], sb);
+                    else if (i == 2) load16_async<64>(dst[rt][i], svoff[rt], sb);
+                    else load16_async<96>(dst[rt][i], svoff[rt], sb);
+                }
+        } else {
+            const uint32_t kc0 = kbeg + last_chunk * BKC;
+#pragma unroll
+            for (int i = 0; i < LPC; ++i) {
+                const uint32_t k = kc0 + 2u * i * EPL;                 // first code of the h = 0 lane load
+                const uint32_t add = k + h * EPL < K ? k * F::bits / 8u : 0u - h * 16u;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) load16_async<0>(dst[rt][i], svoff[rt] + add, a.stream);
             }
         }
     };
-    auto load_thin = [&](uint32_t kc0, uint4 (&dst)[UPT][2]) {
+    u32x4 thin_regs[UPT][2];
+    auto issue_thin = [&](uint32_t ch) {
+        if (ch < last_chunk) {
+            const uint16_t *tb = a.thin + (kbeg + ch * BKC);
 #pragma unroll
-        for (int q = 0; q < UPT; ++q) {
-            const uint32_t u = (uint32_t)t + 256u * q;
-            const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
-            const uint32_t k = kc0 + uc * 16u;
-            const uint32_t c = cbase + row;
+            for (int q = 0; q < UPT; ++q)
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const bool valid = u < (uint32_t)UNITS && c < a.NC && k + 8u * e + 8u <= kend;
-                const uint16_t *src = a.thin + (valid ? (size_t)c * K + k + 8u * e : 0u);
-                const uint32_t keep = valid ? 0xFFFFFFFFu : 0u;
-                uint4 v = *reinterpret_cast<const uint4 *>(src);
-                v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
-                dst[q][e] = v;
+                for (int e = 0; e < 2; ++e) load16_async<0>(thin_regs[q][e], tvoff[q][e], tb);
+        } else {
+            const uint32_t kc0 = kbeg + last_chunk * BKC;
+#pragma unroll
+            for (int q = 0; q < UPT; ++q) {
+                const uint32_t uc = ((uint32_t)t + 256u * q) % (BKC / 16);
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const bool valid = trow_ok[q] && kc0 + uc * 16u + 8u * e + 8u <= kend;
+                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, a.thin);
+                }
             }
         }
     };
-    auto store_thin = [&](int stage, const uint4 (&src)[UPT][2]) {
+    // ties the registers to the preceding wait: nothing that reads them is scheduled above it
+    auto pin_stream = [&](u32x4 (&r)[RT][LPC]) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int i = 0; i < LPC; ++i) asm volatile("" : "+v"(r[rt][i]));
+    };
+    auto pin_thin = [&]() {
+#pragma unroll
+        for (int q = 0; q < UPT; ++q)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) asm volatile("" : "+v"(thin_regs[q][e]));
+    };
+    auto store_thin = [&](int stage, uint32_t ch) {
+        const uint32_t kc0 = kbeg + (ch < last_chunk ? ch : last_chunk) * BKC;
 #pragma unroll
         for (int q = 0; q < UPT; ++q) {
             const uint32_t u = (uint32_t)t + 256u * q;
             if (u >= (uint32_t)UNITS) continue;
             const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
-            const uint32_t in[8] = {src[q][0].x, src[q][0].y, src[q][0].z, src[q][0].w,
-                                    src[q][1].x, src[q][1].y, src[q][1].z, src[q][1].w};
+            const uint32_t k = kc0 + uc * 16u;
+            const uint32_t keep0 = (trow_ok[q] && k + 8u <= kend) ? 0xFFFFFFFFu : 0u;
+            const uint32_t keep1 = (trow_ok[q] && k + 16u <= kend) ? 0xFFFFFFFFu : 0u;
+            const uint32_t in[8] = {thin_regs[q][0].x & keep0, thin_regs[q][0].y & keep0, thin_regs[q][0].z & keep0,
+                                    thin_regs[q][0].w & keep0, thin_regs[q][1].x & keep1, thin_regs[q][1].y & keep1,
+                                    thin_regs[q][1].z & keep1, thin_regs[q][1].w & keep1};
             uint32_t o[8];
 #pragma unroll
             for (int w = 0; w < 8; ++w) {
-                constexpr int dummy = 0; (void)dummy;
                 const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
                 const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
                                      ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
@@ -1712,21 +1764,25 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
         }
     };
 
-    auto compute = [&](int stage, const uint4 (&cur)[RT][LPC]) {
+    auto compute = [&](int stage, uint32_t ch, const u32x4 (&cur)[RT][LPC]) {
         const uint8_t *sbase = sk_lds + stage * STAGE + n31 * PITCH + h * (EPL * 2);
+        const uint32_t kc0 = kbeg + ch * BKC;
 #pragma unroll
         for (int i = 0; i < LPC; ++i) {
+            // 16-bit values past the end of the row could be NaN or infinite: masked (integer codes need not be)
+            const uint32_t keep = (F::bits == 16 && kc0 + (2u * i + h) * EPL >= K) ? 0u : 0xFFFFFFFFu;
 #pragma unroll
             for (int j = 0; j < STEPS; ++j) {
-                constexpr int dummy = 0; (void)dummy;
                 const int koff = (2 * i * EPL + 8 * j) * 2;
                 uint4 tf[CT];
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) tf[ct] = *reinterpret_cast<const uint4 *>(sbase + ct * 32 * PITCH + koff);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
+                    uint4 v = make_uint4(cur[rt][i].x, cur[rt][i].y, cur[rt][i].z, cur[rt][i].w);
+                    if constexpr (F::bits == 16) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
                     uint32_t sf[4];
-                    skinny_frag<FMT>(cur[rt][i], j, sf);
+                    skinny_frag<FMT>(v, j, sf);
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
                         if constexpr (F16T) {
@@ -1745,29 +1801,36 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
             }
         }
     };
-    // one chunk: fetch chunk ch + 1 into `nxt`, multiply chunk ch held in `cur`
-    uint4 thin_regs[UPT][2];
-    auto step = [&](uint32_t ch, const uint4 (&cur)[RT][LPC], uint4 (&nxt)[RT][LPC]) {
+    // One chunk.  In flight on entry: streamed chunks ch (in `cur`) and ch + 1; issued here: the thin block of
+    // ch + 1, then streamed chunk ch + 2 into `far`.  Loads complete in order, so waiting until only the S_LOADS
+    // youngest are outstanding means the thin block (and everything older) has arrived.
+    auto step = [&](uint32_t ch, u32x4 (&cur)[RT][LPC], u32x4 (&far)[RT][LPC]) {
         const int stage = (int)(ch & 1u);
-        const bool more = ch + 1 < nchunks;
-        if (more) {
-            load_stream(kbeg + (ch + 1) * BKC, nxt);
-            load_thin(kbeg + (ch + 1) * BKC, thin_regs);
-        }
-        compute(stage, cur);
-        if (more) store_thin(stage ^ 1, thin_regs);
+        issue_thin(ch + 1);
+        issue_stream(ch + 2, far);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S_LOADS + T_LOADS) : "memory");    // chunk ch is here
+        pin_stream(cur);
+        compute(stage, ch, cur);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S_LOADS) : "memory");
+        pin_thin();
+        store_thin(stage ^ 1, ch + 1);
         __syncthreads();
     };
 
-    uint4 ra[RT][LPC], rb[RT][LPC];
-    load_stream(kbeg, ra);
-    load_thin(kbeg, thin_regs);
-    store_thin(0, thin_regs);
+    u32x4 ra[RT][LPC], rb[RT][LPC], rc[RT][LPC];
+    issue_thin(0);
+    issue_stream(0, ra);
+    issue_stream(1, rb);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S_LOADS) : "memory");
+    pin_thin();
+    store_thin(0, 0);
     __syncthreads();
-    for (uint32_t ch = 0; ch < nchunks; ch += 2) {
-        step(ch, ra, rb);
+    for (uint32_t ch = 0; ch < nchunks; ch += 3) {
+        step(ch, ra, rc);
         if (ch + 1 < nchunks) step(ch + 1, rb, ra);
+        if (ch + 2 < nchunks) step(ch + 2, rc, rb);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the redundant tail loads
 
     // accumulator register r of lane (n31, h): thin row 8 (r / 4) + 4 h + r % 4, streamed row n31
 #pragma unroll
@@ -2276,7 +2339,6 @@ struct ThinPlan {
 ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
 {
     ThinPlan p{};
-    const int wbits = fmt_bits(fmt);
     if (N <= 64 && K % 8u == 0 && M >= 1) {
         p.use = true; p.mode_b = true; p.R = M; p.NC = N;
     } else if (M <= 256 && rows_aligned(fmt, K) && K % 8u == 0) {
@@ -2285,8 +2347,12 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
         return p;
     }
     const int sfmt = p.mode_b ? F16 : fmt;
+    // the kernel addresses both operands with 32-bit lane offsets
+    if ((uint64_t)p.R * K * (uint64_t)fmt_bits(sfmt) / 8u >= (1ull << 32) || (uint64_t)p.NC * K * 2u >= (1ull << 32)) {
+        p.use = false;
+        return p;
+    }
     const uint32_t bkc = sfmt == I8 ? 128u : (sfmt == I4 || sfmt == I2) ? 256u : 64u;
-    (void)wbits;
     p.ct = p.NC <= 32 ? 1 : 2;
     p.cblocks = (p.NC + 32u * p.ct - 1) / (32u * p.ct);
     p.rt = (p.R + 255u) / 256u * p.cblocks >= 128u ? 2 : 1;
