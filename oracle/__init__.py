@@ -42,6 +42,15 @@ class _Net(C.Structure):
 _lib = None
 
 
+class _OptArgs(C.Structure):
+    _fields_ = [("optimizer", C.c_int), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
+                ("momentum", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("epsilon", C.c_float),
+                ("max_grad_norm", C.c_float)]
+
+
+OPT_SGD, OPT_MOMENTUM, OPT_RMSPROP, OPT_ADAM, OPT_ADAMW = range(5)
+
+
 def lib():
     global _lib
     if _lib is not None:
@@ -80,6 +89,15 @@ def lib():
     L.orc_batch_loss.restype = C.c_float
     L.orc_batch_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_int, C.c_int]
     L.orc_argmax.restype = C.c_uint32; L.orc_argmax.argtypes = [C.c_void_p, C.c_uint32]
+    L.orc_derivative.restype = C.c_float; L.orc_derivative.argtypes = [C.c_float, C.c_int]
+    L.orc_batch_gradients.restype = None
+    L.orc_batch_gradients.argtypes = [P(_Net), C.c_void_p, C.c_void_p, C.c_uint32, C.c_float,
+                                      C.c_void_p, C.c_void_p, C.c_void_p]
+    L.orc_clip_grad_norm.restype = C.c_float
+    L.orc_clip_grad_norm.argtypes = [P(_Net), C.c_void_p, C.c_void_p, C.c_float]
+    L.orc_apply_gradients.restype = None
+    L.orc_apply_gradients.argtypes = [P(_Net), P(_OptArgs), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_void_p, C.c_void_p, C.c_float, C.c_float]
     _lib = L
     return L
 
@@ -200,6 +218,30 @@ class Net:
         sec = lib().orc_time_forward_batch(self._h, _ptr(X), X.shape[0], _ptr(out), iters, fn, threads)
         return sec, out
 
+    def batch_gradients(self, X: np.ndarray, T: np.ndarray, grad_scale: float | None = None):
+        """(gW, gB, outputs) of one batch: flat arrays laid out like weights / biases."""
+        X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, self.topology[0])
+        T = np.ascontiguousarray(T, dtype=np.float32).reshape(X.shape[0], self.topology[-1])
+        gW = np.zeros(self.weights.size, dtype=np.float32)
+        gB = np.zeros(self.biases.size, dtype=np.float32)
+        out = np.empty((X.shape[0], self.topology[-1]), dtype=np.float32)
+        scale = 1.0 / X.shape[0] if grad_scale is None else grad_scale
+        lib().orc_batch_gradients(self._h, _ptr(X), _ptr(T), X.shape[0], scale, _ptr(gW), _ptr(gB), _ptr(out))
+        return gW, gB, out
+
+    def clip_grad_norm(self, gW: np.ndarray, gB: np.ndarray, max_norm: float) -> float:
+        return float(lib().orc_clip_grad_norm(self._h, _ptr(gW), _ptr(gB), max_norm))
+
+    def apply_gradients(self, state: "TrainState", gW: np.ndarray, gB: np.ndarray, optimizer: int,
+                        lr: float = 0.01, weight_decay: float = 0.0, momentum: float = 0.9, beta1: float = 0.9,
+                        beta2: float = 0.999, epsilon: float = 1e-8, max_grad_norm: float = 0.0) -> None:
+        """One optimizer step in place (weights, biases, state; gW / gB are modified like the reference's)."""
+        state.beta1_pow *= np.float32(beta1)
+        state.beta2_pow *= np.float32(beta2)
+        a = _OptArgs(optimizer, lr, weight_decay, momentum, beta1, beta2, epsilon, max_grad_norm)
+        lib().orc_apply_gradients(self._h, C.byref(a), _ptr(gW), _ptr(gB), _ptr(state.mW), _ptr(state.vW),
+                                  _ptr(state.mB), _ptr(state.vB), float(state.beta1_pow), float(state.beta2_pow))
+
     def __del__(self):
         try:
             if self._h:
@@ -207,6 +249,24 @@ class Net:
                 self._h = None
         except Exception:
             pass
+
+
+class TrainState:
+    """Optimizer moments of a net plus the running powers beta^t of one train() call (Training.c:684-685)."""
+
+    def __init__(self, net: Net):
+        self.mW = np.zeros(net.weights.size, dtype=np.float32)
+        self.vW = np.zeros(net.weights.size, dtype=np.float32)
+        self.mB = np.zeros(net.biases.size, dtype=np.float32)
+        self.vB = np.zeros(net.biases.size, dtype=np.float32)
+        self.beta1_pow = np.float32(1.0)
+        self.beta2_pow = np.float32(1.0)
+
+
+def derivative(a: np.ndarray, act: int) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    L = lib()
+    return np.array([L.orc_derivative(float(v), act) for v in a.ravel()], dtype=np.float32).reshape(a.shape)
 
 
 def activate(x: np.ndarray, act: int) -> np.ndarray:

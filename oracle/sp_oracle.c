@@ -567,6 +567,171 @@ uint32_t orc_argmax(const float *row, uint32_t width)
 }
 
 
+/* ------------------------------------------------------------------ batched training step */
+/* Activation.c:40-56 (derivative) — the scalar form apply_derivative_batch (SIMD.c:90-188)
+ * multiplies by; its argument is the activation's OUTPUT. */
+float orc_derivative(float a, int act)
+{
+    switch (act) {
+    case ORC_ACT_RELU:       return a > 0.0f ? 1.0f : 0.0f;
+    case ORC_ACT_LEAKY_RELU: return a > 0.0f ? 1.0f : 0.01f;
+    case ORC_ACT_SIGMOID:
+    case ORC_ACT_SOFTMAX:    return a * (1.0f - a);
+    case ORC_ACT_TANH:       return 1.0f - a * a;
+    case ORC_ACT_FOO52:      return (a > 1.0f || a < 0.0f) ? 0.01f : 1.0f;
+    default:                 return 1.0f;
+    }
+}
+
+/* batch_forward keeping every layer (Training.c:313-345 with the BatchWorkspace of :254-311),
+ * batch_compute_deltas (:347-394) and batch_accumulate_gradients (:396-419).  The three matrix
+ * products are summed in double and rounded once (the reference calls sgemm; neither its
+ * blocking nor its summation order is restated).  gW / gB are laid out like weights / biases. */
+void orc_batch_gradients(const orc_net *n, const float *X, const float *T, uint32_t N, float grad_scale,
+                         float *gW, float *gB, float *outputs)
+{
+    const uint32_t last = n->layers - 1;
+    float **act = (float **)calloc(n->layers, sizeof(float *));
+    float **delta = (float **)calloc(n->layers, sizeof(float *));
+    act[0] = (float *)X;
+    for (uint32_t l = 1; l <= last; ++l) {
+        act[l] = (float *)malloc(4u * (size_t)N * n->topology[l]);
+        delta[l] = (float *)malloc(4u * (size_t)N * n->topology[l]);
+    }
+    for (uint32_t l = 1; l <= last; ++l) {
+        const uint32_t in = n->topology[l - 1], o = n->topology[l];
+        const float *W = n->weights + n->woff[l - 1], *b = n->biases + n->boff[l - 1];
+        for (uint64_t s = 0; s < N; ++s)
+            for (uint32_t j = 0; j < o; ++j) {
+                double acc = 0.0;
+                for (uint32_t k = 0; k < in; ++k) acc += (double)act[l - 1][s * in + k] * (double)W[(uint64_t)j * in + k];
+                act[l][s * o + j] = (float)acc + b[j];
+            }
+        orc_apply_activation(act[l], N, o, n->act[l - 1]);
+    }
+    const uint32_t n_out = n->topology[last];
+    const int last_act = n->act[last - 1];
+    if (outputs) memcpy(outputs, act[last], 4u * (size_t)N * n_out);
+
+    /* output layer (Training.c:357-378) */
+    if (n->loss == 0 && last_act == ORC_ACT_SOFTMAX) {
+        for (uint64_t s = 0; s < N; ++s) {
+            const float *a = act[last] + s * n_out, *t = T + s * n_out;
+            float *d = delta[last] + s * n_out;
+            float sum = 0.0f;
+            for (uint32_t j = 0; j < n_out; ++j) sum += (a[j] - t[j]) * a[j];
+            for (uint32_t j = 0; j < n_out; ++j) d[j] = a[j] * ((a[j] - t[j]) - sum);
+        }
+    } else if (n->loss == 1 && (last_act == ORC_ACT_SOFTMAX || last_act == ORC_ACT_SIGMOID)) {
+        for (uint64_t i = 0; i < (uint64_t)N * n_out; ++i) delta[last][i] = act[last][i] + -1.0f * T[i];
+    } else {
+        for (uint64_t i = 0; i < (uint64_t)N * n_out; ++i)
+            delta[last][i] = (act[last][i] - T[i]) * orc_derivative(act[last][i], last_act);
+    }
+    /* hidden layers (Training.c:380-393): delta_l = (delta_{l+1} W_{l+1}) .* f'(act_l) */
+    for (uint32_t l = last - 1; l > 0; --l) {
+        const uint32_t cur = n->topology[l], nxt = n->topology[l + 1];
+        const float *W = n->weights + n->woff[l];
+        for (uint64_t s = 0; s < N; ++s)
+            for (uint32_t k = 0; k < cur; ++k) {
+                double acc = 0.0;
+                for (uint32_t j = 0; j < nxt; ++j) acc += (double)delta[l + 1][s * nxt + j] * (double)W[(uint64_t)j * cur + k];
+                delta[l][s * cur + k] = (float)acc * orc_derivative(act[l][s * cur + k], n->act[l - 1]);
+            }
+    }
+    /* gradients (Training.c:399-418): gW = scale * delta^T act, gB = scale * delta^T ones */
+    for (uint32_t l = 0; l < last; ++l) {
+        const uint32_t in = n->topology[l], o = n->topology[l + 1];
+        float *gw = gW + n->woff[l], *gb = gB + n->boff[l];
+        for (uint32_t j = 0; j < o; ++j) {
+            for (uint32_t k = 0; k < in; ++k) {
+                double acc = 0.0;
+                for (uint64_t s = 0; s < N; ++s) acc += (double)delta[l + 1][s * o + j] * (double)act[l][s * in + k];
+                gw[(uint64_t)j * in + k] = (float)((double)grad_scale * acc);
+            }
+            double accb = 0.0;
+            for (uint64_t s = 0; s < N; ++s) accb += (double)delta[l + 1][s * o + j];
+            gb[j] = (float)((double)grad_scale * accb);
+        }
+    }
+    for (uint32_t l = 1; l <= last; ++l) { free(act[l]); free(delta[l]); }
+    free(act); free(delta);
+}
+
+/* spingalett_clip_grad_norm (SIMD.c:496-520); the squares are added in double here. */
+float orc_clip_grad_norm(const orc_net *n, float *gW, float *gB, float max_norm)
+{
+    if (max_norm <= 0.0f) return 0.0f;
+    double total = 0.0;
+    for (uint64_t i = 0; i < n->total_weights; ++i) total += (double)gW[i] * (double)gW[i];
+    for (uint64_t i = 0; i < n->total_biases; ++i) total += (double)gB[i] * (double)gB[i];
+    const float norm = sqrtf((float)total);
+    if (norm > max_norm) {
+        const float scale = max_norm / norm;
+        for (uint64_t i = 0; i < n->total_weights; ++i) gW[i] *= scale;
+        for (uint64_t i = 0; i < n->total_biases; ++i) gB[i] *= scale;
+    }
+    return norm;
+}
+
+/* one array of apply_gradients_batch_prescaled (Training.c:439-507) with the update rules of
+ * SIMD.c:279-494 in their scalar form; decay is 0 for bias arrays as at the call sites. */
+static void opt_update(const orc_opt_args *a, float *W, float *g, float *m, float *v, uint64_t cnt, float decay,
+                       float beta1_pow_t, float beta2_pow_t)
+{
+    const float lr = a->learning_rate, b1 = a->beta1, b2 = a->beta2, eps = a->epsilon;
+    const float omb1 = 1.0f - b1, omb2 = 1.0f - b2;
+    switch (a->optimizer) {
+    case ORC_OPT_SGD:
+        for (uint64_t i = 0; i < cnt; ++i) {
+            if (decay > 0.0f) W[i] -= lr * (g[i] + decay * W[i]);     /* sgd_decay_update, SIMD.c:401-422 */
+            else W[i] -= lr * g[i];                                   /* sgd_update, :384-399 */
+        }
+        break;
+    case ORC_OPT_MOMENTUM:                                            /* :424-453 */
+        for (uint64_t i = 0; i < cnt; ++i) {
+            m[i] = a->momentum * m[i] + decay * W[i] + g[i];
+            W[i] -= lr * m[i];
+        }
+        break;
+    case ORC_OPT_ADAM:
+    case ORC_OPT_ADAMW: {
+        const float mf = 1.0f / (1.0f - beta1_pow_t), vf = 1.0f / (1.0f - beta2_pow_t);
+        const int adamw = a->optimizer == ORC_OPT_ADAMW;
+        const float wd = (adamw && decay > 0.0f) ? 1.0f - lr * decay : 1.0f;
+        for (uint64_t i = 0; i < cnt; ++i) {
+            if (!adamw && decay > 0.0f) g[i] += decay * W[i];         /* vec_axpy at Training.c:489-491 */
+            m[i] = b1 * m[i] + omb1 * g[i];                           /* adam / adamw update, SIMD.c:279-382 */
+            v[i] = b2 * v[i] + omb2 * (g[i] * g[i]);
+            const float m_hat = m[i] * mf, v_hat = v[i] * vf + eps;
+            if (adamw && decay > 0.0f) W[i] = W[i] * wd - lr * (m_hat / sqrtf(v_hat));
+            else W[i] -= lr * (m_hat / sqrtf(v_hat));
+        }
+        break;
+    }
+    case ORC_OPT_RMSPROP:                                             /* :455-494 */
+        for (uint64_t i = 0; i < cnt; ++i) {
+            v[i] = b2 * v[i] + omb2 * (g[i] * g[i]);
+            const float v_hat = v[i] + eps;
+            W[i] -= lr * (decay * W[i] + g[i] / sqrtf(v_hat));
+        }
+        break;
+    default: break;
+    }
+}
+
+void orc_apply_gradients(orc_net *n, const orc_opt_args *a, float *gW, float *gB, float *mW, float *vW,
+                         float *mB, float *vB, float beta1_pow_t, float beta2_pow_t)
+{
+    if (a->max_grad_norm > 0.0f) orc_clip_grad_norm(n, gW, gB, a->max_grad_norm);
+    for (uint32_t l = 0; l + 1 < n->layers; ++l) {
+        const uint64_t wc = (uint64_t)n->topology[l] * n->topology[l + 1], bc = n->topology[l + 1];
+        const uint64_t wo = n->woff[l], bo = n->boff[l];
+        opt_update(a, n->weights + wo, gW + wo, mW + wo, vW + wo, wc, a->weight_decay, beta1_pow_t, beta2_pow_t);
+        opt_update(a, n->biases + bo, gB + bo, mB + bo, vB + bo, bc, 0.0f, beta1_pow_t, beta2_pow_t);
+    }
+}
+
 double orc_time_forward_batch(const orc_net *n, const float *X, uint32_t N, float *out,
                               int iters, void *sgemm_fn, int threads)
 {

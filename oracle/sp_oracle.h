@@ -26,6 +26,18 @@
  *        vectors, -log of the target's probability for one-hot targets, the
  *        1e-9 clamps at 0 and 1, binary cross-entropy symmetry).
  *   orc_argmax .............................. pinned: numpy argmax (first maximum).
+ *   orc_derivative .......................... pinned: central differences of orc_activate
+ *        away from the kinks, the piecewise constants on either side of them.
+ *   orc_batch_gradients ..................... pinned: central differences in float64 of the
+ *        objective each output-layer rule is the gradient of (half the squared error, or the
+ *        cross-entropy through softmax / sigmoid), weight by weight, on small nets; the bias
+ *        gradient against the gradient of a weight fed by a constant-one input.
+ *   orc_clip_grad_norm ...................... pinned: numpy norm; the norm afterwards equals
+ *        max_norm when it was exceeded and is untouched otherwise.
+ *   orc_apply_gradients ..................... pinned: first-step closed forms (SGD w - lr g;
+ *        Adam and AdamW -lr g / sqrt(g^2 + eps) whatever beta1, beta2; RMSprop
+ *        -lr g / sqrt((1 - beta2) g^2 + eps); momentum's geometric sum over repeated steps
+ *        with a constant gradient), and decay placement per optimizer.
  *   The last-bit summation order of the reference's BLAS / AVX dot product is
  *   deliberately not reproduced (tolerance 1e-4, not bits).
  */
@@ -115,6 +127,26 @@ float orc_batch_loss(const float *outputs, const float *targets, uint32_t N, uin
                      int loss, int output_act);
 /* index of the first largest element of a row (the prediction compared with the label) */
 uint32_t orc_argmax(const float *row, uint32_t width);
+
+/* --- batched training step (Training.c:347-419, 439-507; SIMD.c:279-520) --- */
+enum { ORC_OPT_SGD = 0, ORC_OPT_MOMENTUM, ORC_OPT_RMSPROP, ORC_OPT_ADAM, ORC_OPT_ADAMW };   /* Spingalett.h:76-83 */
+typedef struct {
+    int   optimizer;
+    float learning_rate, weight_decay, momentum, beta1, beta2, epsilon, max_grad_norm;
+} orc_opt_args;
+/* derivative of an activation as a function of its output (Activation.c:40-56) */
+float orc_derivative(float a, int act);
+/* forward keeping all layers, output and hidden deltas, gW = grad_scale * delta^T act and
+ * gB = grad_scale * column sums of delta; gW / gB laid out like weights / biases; outputs
+ * ([N][topology[last]], may be NULL) receives the last layer of the forward. */
+void orc_batch_gradients(const orc_net *net, const float *X, const float *T, uint32_t N, float grad_scale,
+                         float *gW, float *gB, float *outputs);
+/* global L2 norm over gW and gB; both are scaled by max_norm / norm when the norm exceeds it */
+float orc_clip_grad_norm(const orc_net *net, float *gW, float *gB, float max_norm);
+/* one optimizer step over every array of the net (clipping first when max_grad_norm > 0);
+ * beta*_pow_t are beta^t for the step being applied */
+void orc_apply_gradients(orc_net *net, const orc_opt_args *args, float *gW, float *gB, float *mW, float *vW,
+                         float *mB, float *vB, float beta1_pow_t, float beta2_pow_t);
 
 /* CPU-baseline leg: same call sequence with a threaded sgemm.  sgemm_fn is a
  * cblas_sgemm-compatible pointer found at run time, or NULL for the built-in
