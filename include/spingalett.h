@@ -9,8 +9,9 @@
  * unchanged.  The section "additive interface" lists what this build adds;
  * nothing in the reference interface is altered to make room for it.
  *
- * Not provided (outside the inference path): train(), derivative(),
- * print_parameters().
+ * train() runs its two batched strategies on the device; STRATEGY_SAMPLE and
+ * MODE_GENERATOR_FUNCTION are rejected with an error.  Not provided:
+ * derivative(), print_parameters().
  */
 #ifndef SPINGALETT_AMD_H
 #define SPINGALETT_AMD_H
@@ -64,6 +65,13 @@ typedef enum {
     WEIGHT_INITIALIZATION_COUNT
 } WeightInitialization;
 
+/* Spingalett.h:63-83 */
+typedef enum { MODE_ARRAY, MODE_GENERATOR_FUNCTION, MODE_COUNT } TrainingMode;
+typedef enum { STRATEGY_SAMPLE, STRATEGY_FULL_BATCH, STRATEGY_SMALL_BATCH, STRATEGY_COUNT } TrainingStrategy;
+typedef enum {
+    OPTIMIZER_SGD, OPTIMIZER_MOMENTUM, OPTIMIZER_RMSPROP, OPTIMIZER_ADAM, OPTIMIZER_ADAMW, OPTIMIZER_COUNT
+} OptimizerType;
+
 /* Spingalett.h:85-91, with COMPUTE_HIP appended in front of the sentinel.
  * COMPUTE_HIP is the only back-end this library implements; the other
  * values are accepted by spingalett_set_compute_mode() and resolve to
@@ -88,6 +96,9 @@ typedef enum {
     PRECISION_INT2,     /* f32 max | u8[(n+3)/4]  w = q*max, bits 2(i%4)  */
     PRECISION_COUNT
 } PrecisionMode;
+
+/* Spingalett.h:103-107 */
+typedef enum { AUTOSAVE_OFF, AUTOSAVE_OVERWRITE, AUTOSAVE_NEW_FILES } AutoSaveMode;
 
 /* Spingalett.h:109-136.  Plain data, every field readable and writable by
  * the caller.  weights of layer l start at weight_offsets[l] and are
@@ -136,6 +147,45 @@ typedef struct {
     const float *input;
 } ForwardArgs;
 
+/* Spingalett.h:138, 156-189.  Zero fields take the defaults of train_struct_arguments
+ * (Training.c:593-600, 629-632): learning_rate 0.01, momentum 0.9, beta1 0.9, beta2 0.999,
+ * epsilon 1e-8, batch_size 32, callback_interval 1. */
+typedef bool (*TrainCallback)(NeuralNetwork *net, size_t epoch, float current_error);
+typedef struct {
+    NeuralNetwork *net;
+    TrainingMode training_mode;
+    TrainingStrategy training_strategy;
+    OptimizerType optimizer_type;
+
+    float *inputs;               /* [sample_count][topology[0]]    */
+    float *targets;              /* [sample_count][topology[last]] */
+    uint32_t sample_count;
+    uint32_t batch_size;
+    size_t epochs;
+
+    float learning_rate;
+    float weight_decay;
+    float momentum;
+    float beta1;
+    float beta2;
+    float epsilon;
+    float max_grad_norm;
+
+    bool reset_optimizer;
+    size_t nan_check_interval;
+
+    size_t report_interval;
+
+    AutoSaveMode autosave_mode;
+    size_t autosave_interval;
+    const char *autosave_path;
+    bool autosave_do_not_save_optimizer;
+    PrecisionMode autosave_precision;
+
+    TrainCallback callback;
+    size_t callback_interval;
+} TrainArgs;
+
 typedef struct {
     NeuralNetwork *net;
     const char *filename;
@@ -170,6 +220,15 @@ SPINGALETT_API float activate(float x, ActivationFunction act_func);
  * NULL without an error for a NULL net/input, NULL + ERR_INVALID for fewer
  * than two layers or when no GPU can run it. */
 SPINGALETT_API float *forward_struct_arguments(ForwardArgs args);
+/* Spingalett.h:229-230 (Training.c:584-949).  STRATEGY_FULL_BATCH and STRATEGY_SMALL_BATCH run every
+ * step on the device in FP32 (forward keeping all layers, deltas, gradients scaled by 1/batch,
+ * optional clipping by the global norm, SGD / momentum / RMSprop / Adam / AdamW update), with the
+ * reference's epoch loop around them: shuffle per epoch, loss report, NaN check, autosave, callback.
+ * The host arrays (weights, biases, gradients, moments) are current whenever the callback, the NaN
+ * check or autosave look at them and when the call returns; time_step advances once per step.
+ * A net loaded from a quantized file is trained from its FP32 host arrays (what the reference's
+ * loader leaves), and later forwards use the trained FP32 weights.  Errors go to the error slot. */
+SPINGALETT_API void train_struct_arguments(TrainArgs args);
 /* Spingalett.h:232-233 (Serialize.c:307-424) */
 SPINGALETT_API void save_spingalett_struct_arguments(SaveArgs args);
 /* Spingalett.h:235 (Serialize.c:426-609).  Same FP32 host arrays as the
@@ -184,6 +243,7 @@ SPINGALETT_API void free_network(NeuralNetwork *net);
 #define new_spingalett(...)  new_spingalett_struct_arguments((NeuralNetworkArgs){__VA_ARGS__})
 #define layer(...)           layer_struct_arguments((LayerArgs){__VA_ARGS__})
 #define forward(...)         forward_struct_arguments((ForwardArgs){__VA_ARGS__})
+#define train(...)           train_struct_arguments((TrainArgs){__VA_ARGS__})
 #define save_spingalett(...) save_spingalett_struct_arguments((SaveArgs){__VA_ARGS__})
 #endif
 

@@ -92,6 +92,39 @@ SPHIP_API int  sphip_decode(sphip_net *net, uint32_t l, int which, int mode,
 
 SPHIP_API int  sphip_synchronize(void);
 
+/* ---- batched training step (FP32 nets) ----
+ * Takes over what one iteration of the reference's batched epoch loop does between
+ * batch_forward and the end of apply_gradients_batch_prescaled (Training.c:735-748, 769-784):
+ * forward keeping every layer (:313-345), batch_compute_deltas (:347-394),
+ * batch_accumulate_gradients with grad_scale = 1/n (:396-419), optional
+ * spingalett_clip_grad_norm (SIMD.c:496-520) and the optimizer update of every array
+ * (Training.c:439-507, SIMD.c:279-494).  Weights, gradients and moments live on the device
+ * between steps; sphip_train_get copies an array back. */
+typedef struct {
+    int32_t optimizer;      /* OptimizerType (Spingalett.h:76-83): 0 SGD, 1 momentum, 2 RMSprop, 3 Adam,
+                               4 AdamW; negative: gradients only, nothing is updated */
+    int32_t loss_func;      /* LossFunction (Spingalett.h:49-53) */
+    float learning_rate, weight_decay, momentum, beta1, beta2, epsilon;
+    float max_grad_norm;    /* > 0: gradients are scaled to this global L2 norm when they exceed it */
+    float beta1_pow_t, beta2_pow_t;   /* beta^t of the step being applied (Training.c:743-745) */
+} sphip_train_args;
+
+/* arrays of sphip_train_set / sphip_train_get; layer l = 0 .. layers-2, weights row-major [out][in] */
+enum { SPHIP_TRAIN_W = 0, SPHIP_TRAIN_B, SPHIP_TRAIN_MW, SPHIP_TRAIN_VW, SPHIP_TRAIN_MB, SPHIP_TRAIN_VB,
+       SPHIP_TRAIN_GW, SPHIP_TRAIN_GB };
+
+/* Allocates gradients and moments (zeroed).  The net must hold FP32 arrays and no hidden softmax
+ * (train_struct_arguments rejects that too, Training.c:621-627).  Idempotent. */
+SPHIP_API int  sphip_train_begin(sphip_net *net);
+SPHIP_API void sphip_train_end(sphip_net *net);
+SPHIP_API int  sphip_train_set(sphip_net *net, int which, uint32_t l, const float *host);
+SPHIP_API int  sphip_train_get(sphip_net *net, int which, uint32_t l, float *host);
+/* x [n][in], targets [n][out]: host memory, or both device memory with SPHIP_X_ON_DEVICE (then the
+ * call only enqueues).  total_loss, when not NULL, receives batch_compute_loss (Training.c:421-435)
+ * of the forward before the update, and the call waits for it. */
+SPHIP_API int  sphip_train_step(sphip_net *net, const float *x, const float *targets, uint32_t n,
+                                const sphip_train_args *args, uint32_t flags, float *total_loss);
+
 /* ---- measurement helpers (benchmark harness; not part of the data path) ---- */
 SPHIP_API int  sphip_malloc(void **dptr, size_t bytes);
 SPHIP_API int  sphip_free(void *dptr);
@@ -107,6 +140,9 @@ SPHIP_API int  sphip_time_forward(sphip_net *const *nets, int count, const float
 /* Same for the main kernel of one layer only (layer index 1..layers-1). */
 SPHIP_API int  sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer,
                                 uint32_t n, uint32_t flags, int iters, float *ms);
+/* `iters` training steps on device-resident inputs and targets, timed like sphip_time_forward. */
+SPHIP_API int  sphip_time_train_step(sphip_net *net, const float *d_x, const float *d_targets, uint32_t n,
+                                     const sphip_train_args *args, int iters, float *ms);
 /* Name of the main kernel the most recent sphip_time_layer call launched. */
 SPHIP_API const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n,
                                               uint32_t flags);

@@ -31,7 +31,15 @@ SPINGALETT_OK, SPINGALETT_ERR_ALLOC, SPINGALETT_ERR_INVALID = 0, 1, 2
 DEQUANT_STRICT, DEQUANT_RELEASE = 0, 1
 LOG_DEBUG, LOG_INFO, LOG_WARNING, LOG_ERROR, LOG_NONE = range(5)
 
+# Spingalett.h:63-83, 103-107
+MODE_ARRAY, MODE_GENERATOR_FUNCTION = 0, 1
+STRATEGY_SAMPLE, STRATEGY_FULL_BATCH, STRATEGY_SMALL_BATCH = 0, 1, 2
+OPTIMIZER_SGD, OPTIMIZER_MOMENTUM, OPTIMIZER_RMSPROP, OPTIMIZER_ADAM, OPTIMIZER_ADAMW = range(5)
+AUTOSAVE_OFF, AUTOSAVE_OVERWRITE, AUTOSAVE_NEW_FILES = 0, 1, 2
+
 SPHIP_X_ON_DEVICE, SPHIP_Y_ON_DEVICE, SPHIP_FORCE_GEMM, SPHIP_FORCE_GEMV = 1, 2, 8, 16
+(SPHIP_TRAIN_W, SPHIP_TRAIN_B, SPHIP_TRAIN_MW, SPHIP_TRAIN_VW, SPHIP_TRAIN_MB, SPHIP_TRAIN_VB,
+ SPHIP_TRAIN_GW, SPHIP_TRAIN_GB) = range(8)
 
 
 class NeuralNetwork(C.Structure):
@@ -78,6 +86,33 @@ class SaveArgs(C.Structure):
                 ("do_not_save_optimizer", C.c_bool), ("precision", C.c_int)]
 
 
+TrainCallback = C.CFUNCTYPE(C.c_bool, C.POINTER(NeuralNetwork), C.c_size_t, C.c_float)
+
+
+class TrainArgs(C.Structure):
+    """Spingalett.h:156-189, field for field."""
+    _fields_ = [
+        ("net", C.POINTER(NeuralNetwork)), ("training_mode", C.c_int), ("training_strategy", C.c_int),
+        ("optimizer_type", C.c_int),
+        ("inputs", C.POINTER(C.c_float)), ("targets", C.POINTER(C.c_float)),
+        ("sample_count", C.c_uint32), ("batch_size", C.c_uint32), ("epochs", C.c_size_t),
+        ("learning_rate", C.c_float), ("weight_decay", C.c_float), ("momentum", C.c_float),
+        ("beta1", C.c_float), ("beta2", C.c_float), ("epsilon", C.c_float), ("max_grad_norm", C.c_float),
+        ("reset_optimizer", C.c_bool), ("nan_check_interval", C.c_size_t),
+        ("report_interval", C.c_size_t),
+        ("autosave_mode", C.c_int), ("autosave_interval", C.c_size_t), ("autosave_path", C.c_char_p),
+        ("autosave_do_not_save_optimizer", C.c_bool), ("autosave_precision", C.c_int),
+        ("callback", TrainCallback), ("callback_interval", C.c_size_t),
+    ]
+
+
+class SphipTrainArgs(C.Structure):
+    _fields_ = [("optimizer", C.c_int32), ("loss_func", C.c_int32), ("learning_rate", C.c_float),
+                ("weight_decay", C.c_float), ("momentum", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float),
+                ("epsilon", C.c_float), ("max_grad_norm", C.c_float), ("beta1_pow_t", C.c_float),
+                ("beta2_pow_t", C.c_float)]
+
+
 class SphipDesc(C.Structure):
     _fields_ = [("layers", C.c_uint32), ("topology", C.POINTER(C.c_uint32)),
                 ("act", C.POINTER(C.c_uint8)), ("precision", C.c_uint8)]
@@ -96,13 +131,15 @@ PUBLIC_SYMBOLS = [
     "spingalett_set_dequant_mode", "spingalett_get_dequant_mode", "spingalett_forward_batch",
     "spingalett_forward_batch_device", "spingalett_hip_synchronize", "spingalett_hip_invalidate",
     "spingalett_hip_precision", "spingalett_hip_decode", "spingalett_hip_handle", "load_spingalett_memory",
-    "spingalett_evaluate_batch",
+    "spingalett_evaluate_batch", "train_struct_arguments",
 ]
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
     "sphip_forward", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
     "sphip_layer_kernel_name", "sphip_evaluate",
+    "sphip_train_begin", "sphip_train_end", "sphip_train_set", "sphip_train_get", "sphip_train_step",
+    "sphip_time_train_step",
 ]
 
 
@@ -158,6 +195,7 @@ def lib():
     L.spingalett_evaluate_batch.argtypes = [NetPtr, C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(C.c_float),
                                             C.c_void_p, C.POINTER(C.c_uint32)]
     L.spingalett_evaluate_batch.restype = C.c_int
+    L.train_struct_arguments.argtypes = [TrainArgs]; L.train_struct_arguments.restype = None
     L.spingalett_hip_synchronize.restype = C.c_int
     L.spingalett_hip_invalidate.argtypes = [NetPtr]; L.spingalett_hip_invalidate.restype = None
     L.spingalett_hip_precision.argtypes = [NetPtr]; L.spingalett_hip_precision.restype = C.c_int
@@ -189,6 +227,16 @@ def lib():
     L.sphip_time_layer.restype = C.c_int
     L.sphip_layer_kernel_name.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32]
     L.sphip_layer_kernel_name.restype = C.c_char_p
+    L.sphip_train_begin.argtypes = [C.c_void_p]; L.sphip_train_begin.restype = C.c_int
+    L.sphip_train_end.argtypes = [C.c_void_p]; L.sphip_train_end.restype = None
+    L.sphip_train_set.argtypes = [C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]; L.sphip_train_set.restype = C.c_int
+    L.sphip_train_get.argtypes = [C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]; L.sphip_train_get.restype = C.c_int
+    L.sphip_train_step.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(SphipTrainArgs),
+                                   C.c_uint32, C.POINTER(C.c_float)]
+    L.sphip_train_step.restype = C.c_int
+    L.sphip_time_train_step.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(SphipTrainArgs),
+                                        C.c_int, C.POINTER(C.c_float)]
+    L.sphip_time_train_step.restype = C.c_int
     _lib = L
     return L
 
@@ -266,6 +314,32 @@ def evaluate_batch(net, X, T):
         code, msg = last_error()
         raise SpingalettError(f"spingalett_evaluate_batch failed ({code}): {msg}")
     return loss.value, pred, correct.value
+
+
+def train(net, inputs, targets, epochs: int, strategy: int = STRATEGY_FULL_BATCH, optimizer: int = OPTIMIZER_SGD,
+          batch_size: int = 0, callback=None, **kw):
+    """train(...) of the reference (Spingalett.h:229-230); kw: any other TrainArgs field.  Errors are left in
+    the error slot, as there."""
+    X = np.ascontiguousarray(inputs, dtype=np.float32)
+    T = np.ascontiguousarray(targets, dtype=np.float32)
+    n = X.size // net.contents.topology[0]
+    a = TrainArgs()
+    a.net = net
+    a.training_mode = kw.pop("training_mode", MODE_ARRAY)
+    a.training_strategy = strategy
+    a.optimizer_type = optimizer
+    a.inputs = X.ctypes.data_as(C.POINTER(C.c_float))
+    a.targets = T.ctypes.data_as(C.POINTER(C.c_float))
+    a.sample_count = kw.pop("sample_count", n)
+    a.batch_size = batch_size
+    a.epochs = epochs
+    cb = TrainCallback(callback) if callback is not None else TrainCallback()
+    a.callback = cb
+    for k, v in kw.items():
+        if k == "autosave_path" and isinstance(v, str):
+            v = v.encode()
+        setattr(a, k, v)
+    lib().train_struct_arguments(a)
 
 
 def save_spingalett(net, filename: str, precision: int = PRECISION_FLOAT32, do_not_save_optimizer: bool = False):
@@ -420,6 +494,41 @@ class DeviceNet:
         out = np.empty(n, dtype=np.float32)
         _check(lib().sphip_decode(self.h, l, which, mode, out.ctypes.data), "sphip_decode")
         return out
+
+    # ---- batched training step (FP32 nets) ----
+    def train_begin(self):
+        _check(lib().sphip_train_begin(self.h), "sphip_train_begin")
+
+    def train_end(self):
+        lib().sphip_train_end(self.h)
+
+    def _train_count(self, which: int, l: int) -> int:
+        weights = which in (SPHIP_TRAIN_W, SPHIP_TRAIN_MW, SPHIP_TRAIN_VW, SPHIP_TRAIN_GW)
+        return self.topology[l] * self.topology[l + 1] if weights else self.topology[l + 1]
+
+    def train_get(self, which: int, l: int) -> np.ndarray:
+        out = np.empty(self._train_count(which, l), dtype=np.float32)
+        _check(lib().sphip_train_get(self.h, which, l, out.ctypes.data), "sphip_train_get")
+        return out
+
+    def train_set(self, which: int, l: int, values: np.ndarray):
+        v = np.ascontiguousarray(values, dtype=np.float32).ravel()
+        assert v.size == self._train_count(which, l)
+        _check(lib().sphip_train_set(self.h, which, l, v.ctypes.data), "sphip_train_set")
+
+    def train_step(self, X: np.ndarray, T: np.ndarray, args: "SphipTrainArgs", want_loss: bool = False):
+        X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, self.topology[0])
+        T = np.ascontiguousarray(T, dtype=np.float32).reshape(X.shape[0], self.topology[-1])
+        loss = C.c_float(0)
+        _check(lib().sphip_train_step(self.h, X.ctypes.data, T.ctypes.data, X.shape[0], C.byref(args), 0,
+                                      C.byref(loss) if want_loss else None), "sphip_train_step")
+        return loss.value if want_loss else None
+
+    def time_train_step(self, d_x: "DeviceBuffer", d_t: "DeviceBuffer", n: int, args: "SphipTrainArgs", iters: int) -> float:
+        ms = C.c_float(0)
+        _check(lib().sphip_time_train_step(self.h, d_x.ptr, d_t.ptr, n, C.byref(args), iters, C.byref(ms)),
+               "sphip_time_train_step")
+        return ms.value
 
     def destroy(self):
         if self.h and self.owned:

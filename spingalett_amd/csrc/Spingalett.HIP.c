@@ -11,6 +11,7 @@
 #define _GNU_SOURCE
 #include "sp_internal.h"
 
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -212,4 +213,241 @@ void *spingalett_hip_handle(NeuralNetwork *net)
     sp_net *sn = checked(net, "hip_handle");
     if (!sn || !ensure_device(sn)) return NULL;
     return sn->dev;
+}
+
+/* ------------------------------------------------------------------------- *
+ *  train(), Training.c:584-949, for the two batched strategies: the epoch
+ *  loop, reporting, NaN check, autosave and callback run here; each step
+ *  (forward, deltas, gradients, update) runs on the device.
+ * ------------------------------------------------------------------------- */
+static const char *const optimizer_names[] = {"SGD", "MOMENTUM", "RMSPROP", "ADAM", "ADAMW"};
+static const char *const strategy_names[] = {"SGD", "FULL_BATCH", "SMALL_BATCH"};          /* Names.c */
+
+static inline bool should_report(size_t epoch, size_t epochs, size_t interval)      /* Training.c:580-582 */
+{
+    return interval > 0 && ((epoch % interval == 0) || (epoch == epochs));
+}
+
+/* weights, biases, moments and the last gradients back into the host arrays (what the reference's
+ * loop leaves in NeuralNetwork after a step) */
+static bool train_download(sp_net *sn)
+{
+    NeuralNetwork *net = &sn->pub;
+    for (uint32_t l = 0; l + 1 < net->layers; ++l) {
+        const uint64_t wo = net->weight_offsets[l], bo = net->bias_offsets[l];
+        if (sphip_train_get(sn->dev, SPHIP_TRAIN_W, l, net->weights + wo) || sphip_train_get(sn->dev, SPHIP_TRAIN_B, l, net->biases + bo) ||
+            sphip_train_get(sn->dev, SPHIP_TRAIN_MW, l, net->opt_m_weights + wo) || sphip_train_get(sn->dev, SPHIP_TRAIN_VW, l, net->opt_v_weights + wo) ||
+            sphip_train_get(sn->dev, SPHIP_TRAIN_MB, l, net->opt_m_biases + bo) || sphip_train_get(sn->dev, SPHIP_TRAIN_VB, l, net->opt_v_biases + bo) ||
+            sphip_train_get(sn->dev, SPHIP_TRAIN_GW, l, net->grad_weights + wo) || sphip_train_get(sn->dev, SPHIP_TRAIN_GB, l, net->grad_biases + bo)) {
+            report(SPINGALETT_ERR_INVALID, "HIP back-end: train (download)");
+            return false;
+        }
+    }
+    return true;
+}
+
+static bool has_nan_inf(const NeuralNetwork *net)                                    /* Training.c:11-19 */
+{
+    for (uint64_t i = 0; i < net->total_weights; ++i) if (!isfinite(net->weights[i])) return true;
+    for (uint64_t i = 0; i < net->total_biases; ++i) if (!isfinite(net->biases[i])) return true;
+    return false;
+}
+
+static void autosave(NeuralNetwork *net, const TrainArgs *args, size_t epoch)        /* Training.c:536-578 */
+{
+    SaveArgs sa = {.net = net, .do_not_save_optimizer = args->autosave_do_not_save_optimizer, .precision = args->autosave_precision};
+    if (args->autosave_mode == AUTOSAVE_OVERWRITE) {
+        sa.filename = args->autosave_path;
+        save_spingalett_struct_arguments(sa);
+        return;
+    }
+    if (args->autosave_mode != AUTOSAVE_NEW_FILES) return;
+    const char *path = args->autosave_path;
+    const char *dot = strrchr(path, '.'), *slash = strrchr(path, '/'), *back = strrchr(path, '\\');
+    const char *sep = (slash && back) ? (slash > back ? slash : back) : (slash ? slash : back);
+    const bool has_ext = dot && (!sep || dot > sep);
+    const size_t cap = strlen(path) + 64;
+    char *buf = (char *)malloc(cap);
+    if (!buf) return;
+    if (has_ext) snprintf(buf, cap, "%.*s_epoch_%zu%s", (int)(dot - path), path, epoch, dot);
+    else snprintf(buf, cap, "%s_epoch_%zu", path, epoch);
+    sa.filename = buf;
+    save_spingalett_struct_arguments(sa);
+    free(buf);
+}
+
+void train_struct_arguments(TrainArgs args)
+{
+    NeuralNetwork *net = args.net;
+    const uint32_t sample_count = args.sample_count;
+    const size_t epochs = args.epochs;
+
+    /* defaults and checks in the reference's order (Training.c:593-636) */
+    if (args.learning_rate <= 0.0f) args.learning_rate = 0.01f;
+    if (args.momentum <= 0.0f) args.momentum = 0.9f;
+    if (args.beta1 <= 0.0f) args.beta1 = 0.9f;
+    if (args.beta2 <= 0.0f) args.beta2 = 0.999f;
+    if (args.epsilon <= 0.0f) args.epsilon = 1e-8f;
+    if (args.callback && args.callback_interval == 0) args.callback_interval = 1;
+
+    if (args.training_mode == MODE_GENERATOR_FUNCTION) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "Generator function training mode is not implemented yet");
+        sp_log(LOG_ERROR, "Generator function training mode is not implemented yet");
+        return;
+    }
+    if (!net || sample_count == 0 || epochs == 0 || !args.inputs || !args.targets) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "Invalid training arguments (NULL net/inputs/targets or zero count/epochs)");
+        sp_log(LOG_ERROR, "Invalid training arguments");
+        return;
+    }
+    sp_net *sn = checked(net, "train");
+    if (!sn) return;
+    if (net->layers < 2) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "Network must have at least 2 layers for training");
+        sp_log(LOG_ERROR, "Network must have at least 2 layers for training");
+        return;
+    }
+    for (uint32_t l = 1; l + 1 < net->layers; ++l) {
+        if (net->act_func[l - 1] == ACT_SOFTMAX) {
+            sp_set_error(SPINGALETT_ERR_INVALID, "Softmax is not supported in hidden layers");
+            sp_log(LOG_ERROR, "Softmax in hidden layer %u is not supported. Use softmax only in the output layer.", l);
+            return;
+        }
+    }
+    if ((unsigned)args.optimizer_type >= OPTIMIZER_COUNT || (unsigned)args.training_strategy >= STRATEGY_COUNT ||
+        net->loss_func >= LOSS_COUNT) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "Invalid training arguments (unknown optimizer, strategy or loss)");
+        sp_log(LOG_ERROR, "Invalid training arguments");
+        return;
+    }
+    if (args.training_strategy == STRATEGY_SAMPLE) {
+        /* the reference's per-sample loop (Training.c:78-213) is a sequence of single-sample updates;
+         * the device back-end provides the two batched strategies only */
+        sp_set_error(SPINGALETT_ERR_INVALID, "HIP back-end: STRATEGY_SAMPLE is not provided; use STRATEGY_SMALL_BATCH or STRATEGY_FULL_BATCH");
+        sp_log(LOG_ERROR, "HIP back-end: STRATEGY_SAMPLE is not provided; use STRATEGY_SMALL_BATCH or STRATEGY_FULL_BATCH");
+        return;
+    }
+    const bool small = args.training_strategy == STRATEGY_SMALL_BATCH;
+    if (small && args.batch_size == 0) args.batch_size = 32;
+    if (small && args.batch_size > sample_count) args.batch_size = sample_count;
+
+    if (args.reset_optimizer) {                                                      /* Training.c:636-643 */
+        memset(net->opt_m_weights, 0, net->total_weights * sizeof(float));
+        memset(net->opt_v_weights, 0, net->total_weights * sizeof(float));
+        memset(net->opt_m_biases, 0, net->total_biases * sizeof(float));
+        memset(net->opt_v_biases, 0, net->total_biases * sizeof(float));
+        net->time_step = 0;
+        sp_log(LOG_INFO, "Optimizer state reset");
+    }
+    (void)sp_resolve_compute_mode();
+
+    /* training works on the FP32 host arrays: a device copy holding a file's packed arrays is replaced */
+    if (sn->dev && sn->dev_precision != PRECISION_FLOAT32) sp_hip_release(sn);
+    sp_drop_packed(sn);
+    if (sn->dev) sp_hip_release(sn);             /* the host arrays may have been written since the last upload */
+    if (!ensure_device(sn)) return;
+    if (sphip_train_begin(sn->dev)) {
+        report(SPINGALETT_ERR_ALLOC, "HIP back-end: train");
+        return;
+    }
+    for (uint32_t l = 0; l + 1 < net->layers; ++l) {
+        const uint64_t wo = net->weight_offsets[l], bo = net->bias_offsets[l];
+        if (sphip_train_set(sn->dev, SPHIP_TRAIN_MW, l, net->opt_m_weights + wo) || sphip_train_set(sn->dev, SPHIP_TRAIN_VW, l, net->opt_v_weights + wo) ||
+            sphip_train_set(sn->dev, SPHIP_TRAIN_MB, l, net->opt_m_biases + bo) || sphip_train_set(sn->dev, SPHIP_TRAIN_VB, l, net->opt_v_biases + bo)) {
+            report(SPINGALETT_ERR_INVALID, "HIP back-end: train (upload)");
+            sphip_train_end(sn->dev);
+            return;
+        }
+    }
+
+    if (small)
+        sp_log(LOG_INFO, "Starting training: loss=%s, strategy=%s, mode=ARRAY, optimizer=%s, compute=HIP, batch_size=%u",
+               sp_loss_names[net->loss_func], strategy_names[args.training_strategy], optimizer_names[args.optimizer_type], args.batch_size);
+    else
+        sp_log(LOG_INFO, "Starting training: loss=%s, strategy=%s, mode=ARRAY, optimizer=%s, compute=HIP",
+               sp_loss_names[net->loss_func], strategy_names[args.training_strategy], optimizer_names[args.optimizer_type]);
+
+    const uint32_t in_sz = net->topology[0], out_sz = net->topology[net->layers - 1];
+    const uint32_t eff_batch = small ? args.batch_size : sample_count;
+    uint32_t *order = NULL;
+    float *bx = NULL, *bt = NULL;
+    if (small) {
+        order = (uint32_t *)malloc((size_t)sample_count * sizeof(uint32_t));
+        bx = (float *)sp_aligned_calloc((size_t)eff_batch * in_sz, sizeof(float));
+        bt = (float *)sp_aligned_calloc((size_t)eff_batch * out_sz, sizeof(float));
+        if (!order || !bx || !bt) {
+            sp_set_error(SPINGALETT_ERR_ALLOC, "Mini-batch allocation failed");
+            sp_log(LOG_ERROR, "Mini-batch allocation failed");
+            free(order); sp_aligned_free(bx); sp_aligned_free(bt);
+            sphip_train_end(sn->dev);
+            return;
+        }
+        for (uint32_t i = 0; i < sample_count; ++i) order[i] = i;
+    }
+
+    sphip_train_args ta = {
+        .optimizer = (int32_t)args.optimizer_type, .loss_func = (int32_t)net->loss_func,
+        .learning_rate = args.learning_rate, .weight_decay = args.weight_decay, .momentum = args.momentum,
+        .beta1 = args.beta1, .beta2 = args.beta2, .epsilon = args.epsilon, .max_grad_norm = args.max_grad_norm,
+        .beta1_pow_t = 1.0f, .beta2_pow_t = 1.0f,                                   /* Training.c:684-685 */
+    };
+    bool failed = false;
+    for (size_t epoch = 1; epoch <= epochs && !failed; ++epoch) {
+        const bool need_loss = should_report(epoch, epochs, args.report_interval) ||
+                               (args.callback && should_report(epoch, epochs, args.callback_interval));
+        float total_error = 0.0f;
+        if (!small) {
+            float loss = 0.0f;
+            net->time_step++;
+            ta.beta1_pow_t *= args.beta1;
+            ta.beta2_pow_t *= args.beta2;
+            failed = sphip_train_step(sn->dev, args.inputs, args.targets, sample_count, &ta, 0, need_loss ? &loss : NULL) != 0;
+            total_error = loss;
+        } else {
+            sp_shuffle_indices(order, sample_count);
+            for (uint32_t start = 0; start < sample_count && !failed; start += eff_batch) {
+                const uint32_t cur = sample_count - start < eff_batch ? sample_count - start : eff_batch;
+                for (uint32_t s = 0; s < cur; ++s) {                                 /* gather, Training.c:760-767 */
+                    const uint32_t idx = order[start + s];
+                    memcpy(bx + (size_t)s * in_sz, args.inputs + (size_t)idx * in_sz, (size_t)in_sz * sizeof(float));
+                    memcpy(bt + (size_t)s * out_sz, args.targets + (size_t)idx * out_sz, (size_t)out_sz * sizeof(float));
+                }
+                float loss = 0.0f;
+                net->time_step++;
+                ta.beta1_pow_t *= args.beta1;
+                ta.beta2_pow_t *= args.beta2;
+                failed = sphip_train_step(sn->dev, bx, bt, cur, &ta, 0, need_loss ? &loss : NULL) != 0;
+                total_error += loss;
+            }
+        }
+        if (failed) {
+            report(SPINGALETT_ERR_INVALID, "HIP back-end: train (step)");
+            break;
+        }
+        const float current_error = total_error / (float)sample_count;
+        if (should_report(epoch, epochs, args.report_interval))
+            sp_log(LOG_INFO, "Epoch: %zu/%zu, Error: %f", epoch, epochs, (double)current_error);
+
+        /* whoever looks at the host arrays below needs them current */
+        const bool nan_now = args.nan_check_interval > 0 && epoch % args.nan_check_interval == 0;
+        const bool save_now = args.autosave_mode != AUTOSAVE_OFF && args.autosave_interval > 0 && args.autosave_path &&
+                              should_report(epoch, epochs, args.autosave_interval);
+        const bool call_now = args.callback && should_report(epoch, epochs, args.callback_interval);
+        if ((nan_now || save_now || call_now) && !train_download(sn)) break;
+        if (nan_now && has_nan_inf(net)) {
+            sp_log(LOG_ERROR, "NaN/Inf detected in weights at epoch %zu, stopping training", epoch);
+            break;
+        }
+        if (save_now) autosave(net, &args, epoch);
+        if (call_now && args.callback(net, epoch, current_error)) {
+            sp_log(LOG_INFO, "Training interrupted by callback at epoch %zu", epoch);
+            break;
+        }
+    }
+    (void)train_download(sn);
+    sphip_train_end(sn->dev);
+    free(order);
+    sp_aligned_free(bx);
+    sp_aligned_free(bt);
+    sp_log(LOG_INFO, "Training completed.");
 }

@@ -2099,6 +2099,8 @@ struct DevArray {
     bool codes16_valid = false;
 };
 
+struct sphip_train_state;
+
 struct sphip_net {
     uint32_t layers = 0;
     std::vector<uint32_t> topo;
@@ -2129,9 +2131,12 @@ struct sphip_net {
     uint64_t split_cap = 0;
     float *eval_buf = nullptr;     // evaluation: outputs, staged targets, per-sample loss / prediction / hit, totals
     uint64_t eval_cap = 0;
+    sphip_train_state *train = nullptr;   // gradients, optimizer moments, kept activations (training only)
 };
 
 namespace {
+
+void train_free(sphip_net *net);
 
 enum Regime { R_GEMV, R_GEMM16, R_GEMM32 };
 
@@ -2689,6 +2694,7 @@ void sphip_destroy(sphip_net *net)
 {
     if (!net) return;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
+    train_free(net);
     for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); }
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
     if (net->split_ws) (void)hipFree(net->split_ws);
@@ -3002,3 +3008,6 @@ const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, 
 }
 
 }  // extern "C"
+
+// the batched training step (its own kernels and entry points)
+#include "hip_train.inl"

@@ -52,6 +52,8 @@ extern const char *const sp_precision_names[];
 /* sp_network.c */
 NeuralNetwork *sp_net_build(LossFunction loss, uint32_t layers, const uint32_t *topology, const uint8_t *acts);
 
+void sp_shuffle_indices(uint32_t *indices, uint32_t n);
+
 /* sp_format.c */
 size_t sp_array_bytes(uint64_t n, PrecisionMode p);
 /* decodes one serialized array to FP32; returns false if `avail` is too small */

@@ -41,6 +41,17 @@ static uint32_t rng_u32(void)
     return (uint32_t)(r >> 32);
 }
 
+/* Fisher-Yates with the library's generator (spingalett_shuffle_indices, Random.c:73-81) */
+void sp_shuffle_indices(uint32_t *indices, uint32_t n)
+{
+    for (uint32_t i = n; i-- > 1;) {
+        const uint32_t j = rng_u32() % (i + 1);
+        const uint32_t tmp = indices[i];
+        indices[i] = indices[j];
+        indices[j] = tmp;
+    }
+}
+
 static float rng_unit(void) { return (float)(rng_u32() >> 8) * (1.0f / 16777216.0f); }
 
 static float rng_normal(void)

@@ -1,0 +1,292 @@
+"""The batched training step on the device against the oracle's restatement of the reference's
+(Training.c:313-419, 439-507): gradients, every optimizer, clipping, and train() end to end.
+FP32 throughout; tolerance 1e-4 relative to the largest magnitude of the compared array."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as O
+import spingalett_amd as S
+from helpers import make_oracle_net, rel_max_abs
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+
+
+def device_net(onet):
+    d = S.DeviceNet(onet.topology, onet.act, S.PRECISION_FLOAT32)
+    for l in range(onet.layers - 1):
+        d.upload(l, 0, onet.W(l).ravel())
+        d.upload(l, 1, onet.b(l))
+    return d
+
+
+def targets_for(rng, n, width, one_hot):
+    if one_hot:
+        return np.eye(width, dtype=np.float32)[rng.integers(0, width, n)]
+    return rng.uniform(0, 1, (n, width)).astype(np.float32)
+
+
+def step_args(optimizer, loss, **kw):
+    a = S.SphipTrainArgs()
+    a.optimizer = optimizer
+    a.loss_func = loss
+    a.learning_rate = kw.get("lr", 0.01)
+    a.weight_decay = kw.get("weight_decay", 0.0)
+    a.momentum = kw.get("momentum", 0.9)
+    a.beta1 = kw.get("beta1", 0.9)
+    a.beta2 = kw.get("beta2", 0.999)
+    a.epsilon = kw.get("epsilon", 1e-8)
+    a.max_grad_norm = kw.get("max_grad_norm", 0.0)
+    a.beta1_pow_t = 1.0
+    a.beta2_pow_t = 1.0
+    return a
+
+
+GRAD_CASES = [
+    # topology, hidden activations, output activation, loss, batch
+    ([20, 33, 17, 5], ["sigmoid", "tanh"], "softmax", 0, 50),            # vector-path forward, ragged sizes
+    ([20, 33, 17, 5], ["relu", "leaky_relu"], "softmax", 1, 7),
+    ([9, 64, 3], ["foo52"], "sigmoid", 1, 64),
+    ([70, 130, 90, 10], ["tanh", "relu"], "softmax", 1, 300),            # matrix-core forward, K splits everywhere
+    ([70, 130, 90, 10], ["leaky_relu", "sigmoid"], "none", 0, 257),
+    ([64, 128, 64], ["none"], "tanh", 0, 1024),
+    ([5, 3], [], "relu", 1, 33),                                         # single layer, general output rule
+    ([128, 256, 10], ["relu"], "softmax", 1, 1),                         # one sample
+]
+
+
+@pytest.mark.parametrize("topo,hidden,out_act,loss,n", GRAD_CASES)
+def test_gradients_match_oracle(topo, hidden, out_act, loss, n):
+    acts = hidden + [out_act]
+    onet = make_oracle_net(O, topo, acts, seed=len(topo) * 7 + n, bias_std=0.2, loss=loss)
+    rng = np.random.default_rng(n)
+    X = rng.standard_normal((n, topo[0])).astype(np.float32)
+    T = targets_for(rng, n, topo[-1], loss == 1 and out_act in ("softmax", "sigmoid"))
+    gW, gB, out = onet.batch_gradients(X, T)
+    want_loss = O.batch_loss(out, T, loss, O.ACT[out_act])
+
+    d = device_net(onet)
+    d.train_begin()
+    got_loss = d.train_step(X, T, step_args(-1, loss), want_loss=True)
+    assert got_loss == pytest.approx(want_loss, rel=1e-4, abs=1e-5)
+    for l in range(len(topo) - 1):
+        w = gW[onet.woff[l]: onet.woff[l] + topo[l] * topo[l + 1]]
+        b = gB[onet.boff[l]: onet.boff[l] + topo[l + 1]]
+        assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_GW, l), w) <= TOL, l
+        assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_GB, l), b) <= TOL, l
+        # gradients only: nothing moved
+        np.testing.assert_array_equal(d.train_get(S.SPHIP_TRAIN_W, l), onet.W(l).ravel())
+    d.destroy()
+
+
+OPT_CASES = [
+    (S.OPTIMIZER_SGD, {}),
+    (S.OPTIMIZER_SGD, {"weight_decay": 0.3}),
+    (S.OPTIMIZER_MOMENTUM, {"momentum": 0.8, "weight_decay": 0.1}),
+    (S.OPTIMIZER_RMSPROP, {"beta2": 0.9, "epsilon": 1e-6, "weight_decay": 0.05}),
+    (S.OPTIMIZER_ADAM, {}),
+    (S.OPTIMIZER_ADAM, {"weight_decay": 0.2, "beta1": 0.8, "beta2": 0.95}),
+    (S.OPTIMIZER_ADAMW, {"weight_decay": 0.2}),
+    (S.OPTIMIZER_ADAM, {"max_grad_norm": 0.05}),
+    (S.OPTIMIZER_SGD, {"max_grad_norm": 1e6}),                           # norm below the limit: untouched
+]
+
+
+@pytest.mark.parametrize("opt,kw", OPT_CASES)
+def test_four_steps_of_each_optimizer_match_oracle(opt, kw):
+    topo, acts, loss, n = [30, 70, 40, 6], ["tanh", "leaky_relu", "softmax"], 1, 96
+    onet = make_oracle_net(O, topo, acts, seed=opt + 3, bias_std=0.1, loss=loss)
+    rng = np.random.default_rng(opt)
+    X = rng.standard_normal((n, topo[0])).astype(np.float32)
+    T = targets_for(rng, n, topo[-1], True)
+    d = device_net(onet)
+    d.train_begin()
+    st = O.TrainState(onet)
+    a = step_args(opt, loss, lr=0.02, **kw)
+    okw = {"lr": 0.02, **kw}
+    for step in range(4):
+        gW, gB, _ = onet.batch_gradients(X, T)
+        onet.apply_gradients(st, gW, gB, opt, **okw)
+        a.beta1_pow_t = float(st.beta1_pow)
+        a.beta2_pow_t = float(st.beta2_pow)
+        d.train_step(X, T, a)
+        for l in range(len(topo) - 1):
+            assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_W, l), onet.W(l).ravel()) <= TOL, (step, l)
+            assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_B, l), onet.b(l)) <= TOL, (step, l)
+    for l in range(len(topo) - 1):
+        wo, wc = onet.woff[l], topo[l] * topo[l + 1]
+        if opt in (S.OPTIMIZER_MOMENTUM, S.OPTIMIZER_ADAM, S.OPTIMIZER_ADAMW):
+            assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_MW, l), st.mW[wo: wo + wc]) <= TOL
+        if opt in (S.OPTIMIZER_RMSPROP, S.OPTIMIZER_ADAM, S.OPTIMIZER_ADAMW):
+            assert rel_max_abs(d.train_get(S.SPHIP_TRAIN_VW, l), st.vW[wo: wo + wc]) <= 2 * TOL
+    d.destroy()
+
+
+def test_moments_can_be_seeded_and_read_back():
+    onet = make_oracle_net(O, [6, 9, 4], ["relu", "none"])
+    d = device_net(onet)
+    d.train_begin()
+    rng = np.random.default_rng(0)
+    for which in (S.SPHIP_TRAIN_MW, S.SPHIP_TRAIN_VW, S.SPHIP_TRAIN_MB, S.SPHIP_TRAIN_VB):
+        for l in range(2):
+            v = rng.standard_normal(54 if which in (S.SPHIP_TRAIN_MW, S.SPHIP_TRAIN_VW) and l == 0 else
+                                    36 if which in (S.SPHIP_TRAIN_MW, S.SPHIP_TRAIN_VW) else (9, 4)[l]).astype(np.float32)
+            d.train_set(which, l, v)
+            np.testing.assert_array_equal(d.train_get(which, l), v)
+    d.destroy()
+
+
+def test_step_argument_checks():
+    onet = make_oracle_net(O, [6, 9, 4], ["relu", "none"])
+    d = device_net(onet)
+    X, T = np.zeros((2, 6), np.float32), np.zeros((2, 4), np.float32)
+    with pytest.raises(S.SpingalettError, match="sphip_train_begin"):
+        d.train_step(X, T, step_args(0, 0))
+    d.train_begin()
+    with pytest.raises(S.SpingalettError, match="optimizer"):
+        d.train_step(X, T, step_args(9, 0))
+    d.destroy()
+    # packed formats cannot be trained in place, hidden softmax is rejected as in the reference
+    q = S.DeviceNet([4, 4], [S.ACT_NONE], S.PRECISION_INT8)
+    q.upload(0, 0, np.zeros(16, np.uint8), 1.0)
+    q.upload(0, 1, np.zeros(4, np.uint8), 1.0)
+    with pytest.raises(S.SpingalettError, match="FP32"):
+        q.train_begin()
+    q.destroy()
+    sm = device_net(make_oracle_net(O, [4, 5, 3], ["softmax", "none"]))
+    with pytest.raises(S.SpingalettError, match="softmax"):
+        sm.train_begin()
+    sm.destroy()
+
+
+# ------------------------------------------------------------------ train() through the public interface
+def public_net(topo, acts, loss, seed=0):
+    onet = make_oracle_net(O, topo, acts, seed=seed, bias_std=0.1, loss=loss)
+    net = S.new_spingalett(loss)
+    S.layer(net, topo[0], 0, S.WEIGHT_INITIALIZATION_NONE)
+    for l in range(1, len(topo)):
+        S.layer(net, topo[l], O.ACT[acts[l - 1]], S.WEIGHT_INITIALIZATION_NONE)
+    for l in range(len(topo) - 1):
+        S.weights_view(net, l)[:] = onet.W(l)
+        S.biases_view(net, l)[:] = onet.b(l)
+    return net, onet
+
+
+def test_full_batch_train_matches_oracle_epochs():
+    topo, acts, loss, n, epochs = [12, 40, 8, 3], ["tanh", "relu", "softmax"], 1, 150, 6
+    net, onet = public_net(topo, acts, loss, seed=5)
+    rng = np.random.default_rng(1)
+    X = rng.standard_normal((n, topo[0])).astype(np.float32)
+    T = targets_for(rng, n, topo[-1], True)
+    seen = []
+    S.clear_error()
+    S.train(net, X, T, epochs, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.01,
+            callback=lambda p, epoch, err: seen.append((epoch, err)) or False, callback_interval=2)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    st = O.TrainState(onet)
+    want_err = {}
+    for epoch in range(1, epochs + 1):
+        gW, gB, out = onet.batch_gradients(X, T)
+        want_err[epoch] = O.batch_loss(out, T, loss, O.ACT["softmax"]) / n
+        onet.apply_gradients(st, gW, gB, O.OPT_ADAM, lr=0.01)
+    for l in range(len(topo) - 1):
+        assert rel_max_abs(S.weights_view(net, l), onet.W(l)) <= TOL
+        assert rel_max_abs(S.biases_view(net, l), onet.b(l)) <= TOL
+    assert [e for e, _ in seen] == [2, 4, 6]
+    for e, err in seen:
+        assert err == pytest.approx(want_err[e], rel=1e-4)
+    assert net.contents.time_step == epochs
+    # moments came back too (they are what a later save with the optimizer block writes)
+    mw = np.ctypeslib.as_array(net.contents.opt_m_weights, shape=(int(net.contents.total_weights),))
+    assert rel_max_abs(mw, st.mW) <= TOL
+    # and forward() now runs the trained weights
+    y = S.forward_batch(net, X[:5])
+    assert rel_max_abs(y, onet.forward_batch(X[:5])) <= TOL
+    S.free_network(net)
+
+
+def test_small_batch_train_learns_xor_and_counts_steps():
+    """The reference's sanity problem (Examples/XOR.c:20-64)."""
+    net, _ = public_net([2, 8, 1], ["tanh", "sigmoid"], 0, seed=4)
+    X = np.float32([[0, 0], [0, 1], [1, 0], [1, 1]] * 8)
+    T = np.float32([[0], [1], [1], [0]] * 8)
+    errs = []
+    S.clear_error()
+    S.train(net, X, T, 150, S.STRATEGY_SMALL_BATCH, S.OPTIMIZER_ADAM, batch_size=12, learning_rate=0.05,
+            callback=lambda p, epoch, err: errs.append(err) or False, callback_interval=1)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    assert net.contents.time_step == 150 * 3                   # 32 samples in batches of 12: 3 steps per epoch
+    assert errs[-1] < 0.05 * errs[0]
+    y = S.forward_batch(net, X[:4])
+    np.testing.assert_array_equal(y[:, 0] > 0.5, T[:4, 0] > 0.5)
+    S.free_network(net)
+
+
+def test_callback_stops_training_and_autosave_writes_files(tmp_path):
+    net, _ = public_net([4, 6, 2], ["relu", "none"], 0)
+    rng = np.random.default_rng(0)
+    X = rng.standard_normal((10, 4)).astype(np.float32)
+    T = rng.standard_normal((10, 2)).astype(np.float32)
+    path = str(tmp_path / "auto.nn")
+    S.clear_error()
+    S.train(net, X, T, 10, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_SGD, callback=lambda p, epoch, err: epoch == 4,
+            autosave_mode=S.AUTOSAVE_NEW_FILES, autosave_interval=2, autosave_path=path,
+            autosave_precision=S.PRECISION_FLOAT32)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    assert net.contents.time_step == 4
+    assert sorted(os.listdir(tmp_path)) == ["auto_epoch_2.nn", "auto_epoch_4.nn"]
+    # the file holds the weights of that epoch: reloading the last one gives the net as it stands
+    again = S.load_spingalett(str(tmp_path / "auto_epoch_4.nn"))
+    np.testing.assert_array_equal(S.weights_view(again, 0), S.weights_view(net, 0))
+    S.free_network(again)
+    S.free_network(net)
+
+
+def test_train_rejects_what_the_reference_rejects():
+    net, _ = public_net([4, 6, 2], ["softmax", "none"], 0)
+    X, T = np.zeros((3, 4), np.float32), np.zeros((3, 2), np.float32)
+    S.clear_error()
+    S.train(net, X, T, 1)
+    assert S.last_error() == (S.SPINGALETT_ERR_INVALID, "Softmax is not supported in hidden layers")
+    S.free_network(net)
+    net, _ = public_net([4, 6, 2], ["relu", "none"], 0)
+    w0 = S.weights_view(net, 0).copy()
+    for kw, msg in (({"training_mode": S.MODE_GENERATOR_FUNCTION}, "Generator function"),
+                    ({"sample_count": 0}, "Invalid training arguments"),
+                    ({"strategy": S.STRATEGY_SAMPLE}, "STRATEGY_SAMPLE")):
+        S.clear_error()
+        S.train(net, X, T, 1, **kw)
+        code, text = S.last_error()
+        assert code == S.SPINGALETT_ERR_INVALID and msg in text, (kw, text)
+    S.clear_error()
+    S.train(net, X, T, 0)
+    assert S.last_error()[0] == S.SPINGALETT_ERR_INVALID
+    np.testing.assert_array_equal(S.weights_view(net, 0), w0)
+    S.free_network(net)
+
+
+def test_training_a_quantized_net_continues_from_its_fp32_arrays():
+    onet = make_oracle_net(O, [16, 32, 4], ["relu", "softmax"], seed=9, loss=1)
+    blob = onet.serialize(O.PREC["i8"])
+    ref = O.Net.parse(blob)                                    # what the loader's FP32 arrays hold
+    ref.c.loss = 1
+    net = S.load_spingalett_memory(blob)
+    rng = np.random.default_rng(2)
+    X = rng.standard_normal((80, 16)).astype(np.float32)
+    T = targets_for(rng, 80, 4, True)
+    S.forward_batch(net, X)                                    # device copy holds the INT8 arrays now
+    assert S.lib().spingalett_hip_precision(net) == S.PRECISION_INT8
+    S.clear_error()
+    S.train(net, X, T, 2, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_SGD, learning_rate=0.1)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    st = O.TrainState(ref)
+    for _ in range(2):
+        gW, gB, _ = ref.batch_gradients(X, T)
+        ref.apply_gradients(st, gW, gB, O.OPT_SGD, lr=0.1)
+    assert rel_max_abs(S.weights_view(net, 0), ref.W(0)) <= TOL
+    assert S.lib().spingalett_hip_precision(net) == S.PRECISION_FLOAT32
+    assert rel_max_abs(S.forward_batch(net, X), ref.forward_batch(X)) <= TOL
+    S.free_network(net)
