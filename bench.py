@@ -8,7 +8,9 @@ whose weights were written by the library's own serializer and loaded back
 (load_spingalett keeps the packed arrays; the device computes on them).
 Inputs and outputs are device-resident during the timed region.  One JSON line
 is printed: the headline workload plus, under "workloads", the other
-BASELINE configurations with their own roofline figures.
+BASELINE configurations with their own roofline figures and, under "training",
+the reference's published training benchmark (--workload T1 makes that the
+headline instead).
 """
 from __future__ import annotations
 
@@ -251,6 +253,71 @@ def run_workload(name, batches, steps, warmup, want_output=False):
     return dict(net=net, path=path, copies=copies, clones=clones, rows=rows, build_s=build_s)
 
 
+# The reference's own published benchmark (Examples/Benchmark.c:14-98, README.md:48-59): train() on
+# 784 -> 512 ReLU -> 1000 ReLU -> 10 softmax, 20,000 samples, full batch, Adam 0.001, cross-entropy,
+# inputs and targets uniform in [0, 1).
+TRAIN_TOPO = [784, 512, 1000, 10]
+TRAIN_SAMPLES = 20000
+TRAIN_PUBLISHED = dict(value=88921.0, unit="samples/s", hardware="Intel i7-12650H, OpenBLAS, 12 threads", source="README.md:57")
+
+
+def train_flops(n):
+    """2 n (in out) per layer for the forward and for the weight gradients, and for the hidden deltas of layers 2.."""
+    t = TRAIN_TOPO
+    fwd = sum(t[l] * t[l + 1] for l in range(len(t) - 1))
+    return 2 * n * (2 * fwd + sum(t[l] * t[l + 1] for l in range(1, len(t) - 1)))
+
+
+def run_training(steps, warmup, cpu=True):
+    rng = np.random.default_rng(42)
+    t = TRAIN_TOPO
+    acts = [S.ACT_RELU, S.ACT_RELU, S.ACT_SOFTMAX]
+    W = [(rng.standard_normal((t[l + 1], t[l])) * np.sqrt((2.0 if l < 2 else 1.0) / t[l])).astype(np.float32) for l in range(3)]
+    X = rng.random((TRAIN_SAMPLES, t[0]), dtype=np.float32)
+    T = rng.random((TRAIN_SAMPLES, t[-1]), dtype=np.float32)
+    d = S.DeviceNet(t, acts, S.PRECISION_FLOAT32)
+    for l in range(3):
+        d.upload(l, 0, W[l].ravel())
+        d.upload(l, 1, np.zeros(t[l + 1], np.float32))
+    d.train_begin()
+    a = S.SphipTrainArgs(S.OPTIMIZER_ADAM, S.LOSS_CROSS_ENTROPY, 0.001, 0.0, 0.9, 0.9, 0.999, 1e-8, 0.0, 0.9, 0.999)
+    dx, dt = S.DeviceBuffer.from_numpy(X), S.DeviceBuffer.from_numpy(T)
+    d.time_train_step(dx, dt, TRAIN_SAMPLES, a, max(1, warmup))
+    ms = d.time_train_step(dx, dt, TRAIN_SAMPLES, a, steps) / steps
+    finite = bool(np.isfinite(d.train_get(S.SPHIP_TRAIN_W, 0)).all())
+    d.destroy(); dx.free(); dt.free()
+    # the public call as the reference's example times it: host arrays in, trained host arrays out, 5 epochs
+    net = S.new_spingalett(S.LOSS_CROSS_ENTROPY)
+    S.layer(net, t[0], 0, S.WEIGHT_INITIALIZATION_NONE)
+    for l in range(3):
+        S.layer(net, t[l + 1], acts[l], S.WEIGHT_INITIALIZATION_NONE)
+        S.weights_view(net, l)[:] = W[l]
+    S.train(net, X, T, 1, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.001)      # warm-up
+    t0 = time.perf_counter()
+    S.train(net, X, T, 5, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.001)
+    call_s = time.perf_counter() - t0
+    S.free_network(net)
+    out = dict(workload=f"T1: {'->'.join(map(str, t))} FP32, full batch of {TRAIN_SAMPLES}, Adam, cross-entropy "
+                        "(Examples/Benchmark.c)", samples_per_s=TRAIN_SAMPLES / (ms * 1e-3), ms_per_step=ms, steps=steps,
+               fp32_mfma_frac=train_flops(TRAIN_SAMPLES) / (ms * 1e-3) / FP32_PEAK, finite=finite,
+               train_call_samples_per_s=5 * TRAIN_SAMPLES / call_s,
+               published=TRAIN_PUBLISHED, vs_published=TRAIN_SAMPLES / (ms * 1e-3) / TRAIN_PUBLISHED["value"])
+    if cpu:
+        import oracle as O
+        n = 256
+        onet = O.Net.new(t, acts, 1)
+        for l in range(3):
+            onet.W(l)[:] = W[l]
+        st = O.TrainState(onet)
+        t1 = time.perf_counter()
+        gW, gB, _ = onet.batch_gradients(X[:n], T[:n])
+        onet.apply_gradients(st, gW, gB, O.OPT_ADAM, lr=0.001)
+        sec = time.perf_counter() - t1
+        out["cpu_baseline"] = dict(value=n / sec, unit="samples/s", cores=1, kind="port",
+                                   sample=f"one step on {n} samples, scalar restatement (no BLAS)")
+    return out
+
+
 def release(w):
     for hc in w["clones"]:
         S.lib().sphip_destroy(hc)
@@ -267,7 +334,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="C4", choices=sorted(WORKLOADS) + ["T1"],
+                    help="C1..C5: forward configurations; T1: the reference's published training benchmark")
     ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -283,6 +351,18 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
 
+    if args.workload == "T1":
+        tr = run_training(args.steps, args.warmup, cpu=not args.no_cpu)
+        print(json.dumps({
+            "metric": "training samples/sec (forward + backward + Adam), the reference's published benchmark",
+            "value": tr["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": tr["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": tr["vs_published"], "dtype": "fp32", "data": "synthetic (seeded, as Examples/Benchmark.c draws them)",
+            "config": {"workload": tr["workload"]},
+            "roofline": {"bound": "mfma", "achieved": train_flops(TRAIN_SAMPLES) / (tr["ms_per_step"] * 1e-3) / 1e12,
+                         "peak": FP32_PEAK / 1e12, "unit": "TFLOP/s", "frac": tr["fp32_mfma_frac"], "traffic": None},
+            "cpu_baseline": tr.get("cpu_baseline"), "training": tr}))
+        return 0
     cfg = WORKLOADS[args.workload]
     n = args.batch or max(cfg["batches"])
     head = run_workload(args.workload, [n], args.steps, args.warmup)
@@ -313,6 +393,13 @@ def main():
             except Exception as e:  # keep the headline even if an extra configuration fails
                 extra.append(dict(workload=name, error=str(e)))
 
+    training = None
+    if not args.no_extra:
+        try:
+            training = run_training(20, 3, cpu=not args.no_cpu)
+        except Exception as e:
+            training = dict(workload="T1", error=str(e))
+
     rl = dict(row["roofline"])
     out = {
         "metric": "forward samples/sec per weight format; % peak HBM BW (b=1), % MFMA peak (b>=4K)",
@@ -327,6 +414,7 @@ def main():
         "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
         "cpu_baseline": cpu,
         "workloads": extra,
+        "training": training,
     }
     print(json.dumps(out))
     return 0

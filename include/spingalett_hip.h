@@ -39,6 +39,7 @@ typedef struct {
 /* flags of sphip_forward */
 #define SPHIP_X_ON_DEVICE   1u   /* x is a device pointer                       */
 #define SPHIP_Y_ON_DEVICE   2u   /* y is a device pointer (call does not wait)  */
+#define SPHIP_TRAIN_SAME_BATCH 4u /* sphip_train_step: reuse the host batch the previous step copied in */
 #define SPHIP_FORCE_GEMM    8u   /* use the matrix-core path whatever n is      */
 #define SPHIP_FORCE_GEMV   16u   /* use the vector path (n <= 64)               */
 
@@ -120,7 +121,8 @@ SPHIP_API void sphip_train_end(sphip_net *net);
 SPHIP_API int  sphip_train_set(sphip_net *net, int which, uint32_t l, const float *host);
 SPHIP_API int  sphip_train_get(sphip_net *net, int which, uint32_t l, float *host);
 /* x [n][in], targets [n][out]: host memory, or both device memory with SPHIP_X_ON_DEVICE (then the
- * call only enqueues).  total_loss, when not NULL, receives batch_compute_loss (Training.c:421-435)
+ * call only enqueues); with SPHIP_TRAIN_SAME_BATCH x and targets are ignored and the batch of the
+ * previous host-memory step (same n) is used again without a copy.  total_loss, when not NULL, receives batch_compute_loss (Training.c:421-435)
  * of the forward before the update, and the call waits for it. */
 SPHIP_API int  sphip_train_step(sphip_net *net, const float *x, const float *targets, uint32_t n,
                                 const sphip_train_args *args, uint32_t flags, float *total_loss);

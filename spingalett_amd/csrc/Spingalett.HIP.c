@@ -401,7 +401,9 @@ void train_struct_arguments(TrainArgs args)
             net->time_step++;
             ta.beta1_pow_t *= args.beta1;
             ta.beta2_pow_t *= args.beta2;
-            failed = sphip_train_step(sn->dev, args.inputs, args.targets, sample_count, &ta, 0, need_loss ? &loss : NULL) != 0;
+            /* the batch is the same every epoch: it crosses PCIe once */
+            failed = sphip_train_step(sn->dev, args.inputs, args.targets, sample_count, &ta,
+                                      epoch == 1 ? 0u : SPHIP_TRAIN_SAME_BATCH, need_loss ? &loss : NULL) != 0;
             total_error = loss;
         } else {
             sp_shuffle_indices(order, sample_count);

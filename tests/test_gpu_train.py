@@ -53,6 +53,7 @@ GRAD_CASES = [
     ([70, 130, 90, 10], ["tanh", "relu"], "softmax", 1, 300),            # matrix-core forward, K splits everywhere
     ([70, 130, 90, 10], ["leaky_relu", "sigmoid"], "none", 0, 257),
     ([64, 128, 64], ["none"], "tanh", 0, 1024),
+    ([390, 520, 300, 10], ["tanh", "relu"], "softmax", 1, 700),          # ragged edges in every product
     ([5, 3], [], "relu", 1, 33),                                         # single layer, general output rule
     ([128, 256, 10], ["relu"], "softmax", 1, 1),                         # one sample
 ]
