@@ -77,10 +77,7 @@ int fail_hip(const char *what, hipError_t e)
 
 hipStream_t g_stream = nullptr;
 const char *g_last_kernel = "";   // main kernel of the most recent layer launch
-int g_gemv_variant = 1;     // 0: vector-ALU GEMV only (tuning switch)
-int g_gemv_waves = 0;       // 0: automatic
-int g_gemv_lds_kib = 64;
-int g_gemm_variant = 1;     // 0: 128x128 tiles only (tuning switch)
+constexpr uint32_t kGemvStageBytes = 64u * 1024u;   // LDS budget of one stage of the integer GEMV
 
 std::mutex g_init_mutex;
 
@@ -94,10 +91,6 @@ int ensure_stream()
     if (cnt <= 0) return fail_msg("no HIP device");
     HCHECK(hipSetDevice(0));
     HCHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
-    if (const char *v = getenv("SPHIP_GEMM_VARIANT")) g_gemm_variant = atoi(v);
-    if (const char *v = getenv("SPHIP_GEMV_VARIANT")) g_gemv_variant = atoi(v);
-    if (const char *v = getenv("SPHIP_GEMV_WAVES")) g_gemv_waves = atoi(v);
-    if (const char *v = getenv("SPHIP_GEMV_LDS")) g_gemv_lds_kib = atoi(v);
     return 0;
 }
 
@@ -2205,7 +2198,7 @@ template <int FMT>
 bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
 {
     constexpr int KL = I8Fmt<FMT>::KL;
-    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq || g_gemv_variant == 0) return false;
+    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq) return false;
     if (reinterpret_cast<uintptr_t>(x) & 15u) return false;   // the quantiser reads float4
     const int need = (int)(n + 3) / 4;
     const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
@@ -2216,10 +2209,10 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     const uint32_t wave_rows = (L.N + 15) / 16;
     const uint32_t kblocks = (L.K + KL - 1) / KL;
     const uint32_t blk_bytes = (uint32_t)I8Fmt<FMT>::NMF * 4u * n * 48u;
-    const uint32_t budget = (uint32_t)g_gemv_lds_kib * 1024u;
+    const uint32_t budget = kGemvStageBytes;
     const uint32_t max_waves = MT > 4 ? 4u : 16u;             // register budget of the wide tiles
     // up to four samples: the GEMV workgroups quantise the activations themselves
-    const bool fused = MT == 1 && g_gemv_variant != 2;
+    const bool fused = MT == 1;
     const uint32_t ks_cap = 2048u / (4u * KL);                 // a scale chunk is a whole number of fetch groups
                                                                // and at most 2048 codes (one wave's batch of loads)
     uint32_t rw, ks;
@@ -2239,11 +2232,6 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
         while (rw > 1 && wave_rows / rw < 512u) rw >>= 1;      // keep the grid at least twice the chip
         ks = max_waves / rw > 8u ? 8u : max_waves / rw;
         if (ks > ks_cap) ks = ks_cap;
-    }
-    if (g_gemv_waves) {
-        rw = (uint32_t)g_gemv_waves & 15u; ks = (uint32_t)g_gemv_waves >> 4;
-        if (ks > ks_cap) ks = ks_cap;
-        while (fused && rw * ks > 8u) rw >>= 1;
     }
     // one fetch group (4 blocks of every K share) must fit the row, the stage budget and one scale chunk
     while (ks > 1 && (kblocks < 4u * ks || 4u * ks * blk_bytes > budget)) ks >>= 1;
@@ -2402,7 +2390,7 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
 template <int FMT, bool F16T>
 void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
 {
-    const ThinPlan tp = g_gemm_variant == 4 ? ThinPlan{} : plan_thin(FMT, M, L.N, L.K);
+    const ThinPlan tp = plan_thin(FMT, M, L.N, L.K);
     if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
         a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
@@ -2424,9 +2412,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
     const uint32_t big_tiles = ((M + 255u) / 256u) * ((L.N + 255u) / 256u);
     const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
-    const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats && g_gemm_variant != 7;
-    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && g_gemm_variant != 0 &&
-        (big_tiles >= 192u || split_ok || g_gemm_variant == 5)) {
+    const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
+    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
         constexpr int BM = 256, BN = 256;
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
         else g.ws = ctx.ws;
