@@ -291,3 +291,37 @@ def test_training_a_quantized_net_continues_from_its_fp32_arrays():
     assert S.lib().spingalett_hip_precision(net) == S.PRECISION_FLOAT32
     assert rel_max_abs(S.forward_batch(net, X), ref.forward_batch(X)) <= TOL
     S.free_network(net)
+
+
+def test_full_size_benchmark_step_properties():
+    """The reference's benchmark net at its full batch (Examples/Benchmark.c: 784-512-1000-10, 20,000 samples), through
+    properties that do not need the oracle at that size: the gradient of the whole batch is the mean of the gradients
+    of its two halves, the reported loss is the sum of the halves' losses, and Adam steps lower the loss of one-hot targets."""
+    topo, n = [784, 512, 1000, 10], 20000
+    rng = np.random.default_rng(3)
+    d = S.DeviceNet(topo, [S.ACT_RELU, S.ACT_RELU, S.ACT_SOFTMAX], S.PRECISION_FLOAT32)
+    for l in range(3):
+        std = np.sqrt((2.0 if l < 2 else 1.0) / topo[l])
+        d.upload(l, 0, (rng.standard_normal(topo[l] * topo[l + 1]) * std).astype(np.float32))
+        d.upload(l, 1, np.zeros(topo[l + 1], np.float32))
+    X = rng.random((n, topo[0]), dtype=np.float32)
+    T = rng.random((n, topo[-1]), dtype=np.float32)
+    d.train_begin()
+    grads = {}
+    losses = {}
+    for name, sl in (("all", slice(0, n)), ("a", slice(0, n // 2)), ("b", slice(n // 2, n))):
+        losses[name] = d.train_step(X[sl], T[sl], step_args(-1, 1), want_loss=True)
+        grads[name] = [d.train_get(S.SPHIP_TRAIN_GW, l) for l in range(3)] + [d.train_get(S.SPHIP_TRAIN_GB, l) for l in range(3)]
+    assert losses["all"] == pytest.approx(losses["a"] + losses["b"], rel=1e-5)
+    for g_all, g_a, g_b in zip(grads["all"], grads["a"], grads["b"]):
+        assert np.isfinite(g_all).all()
+        assert rel_max_abs(g_all, 0.5 * (g_a.astype(np.float64) + g_b)) <= TOL
+    # descent needs targets the output rule is the gradient for (rows that sum to 1; the benchmark's uniform targets do not)
+    hot = np.eye(topo[-1], dtype=np.float32)[rng.integers(0, topo[-1], n)]
+    a = step_args(S.OPTIMIZER_ADAM, 1, lr=0.001)
+    seen = []
+    for step in range(1, 7):
+        a.beta1_pow_t, a.beta2_pow_t = 0.9 ** step, 0.999 ** step
+        seen.append(d.train_step(X, hot, a, want_loss=True))
+    assert seen[-1] < seen[0]
+    d.destroy()
