@@ -1,12 +1,16 @@
 // hip_forward.hip — gfx950 kernels and the C ABI of spingalett_hip.h.
 //
-// One translation unit holds every HIP runtime call and every kernel of the
-// inference path:
-//   sp_decode_*      element decoders (bit-exact with Serialize.c:45-85,195-297)
-//   sp_gemv_*        n <= 64: FP32-arithmetic dequant GEMV, fused bias+activation
-//   sp_gemm16_*      n  > 64: LDS-tiled dequant-to-16-bit MFMA GEMM, fused epilogue
-//   sp_gemm32_f32    n  > 64 with FP32 weights: FP32 MFMA GEMM
-//   sp_softmax_rows  per-sample softmax (Activation.c:5-21)
+// One translation unit holds every HIP runtime call and every kernel:
+//   sp_decode         element decoders (bit-exact with Serialize.c:45-85,195-297)
+//   sp_gemv*          1..4 samples (FP32 weights: up to 64): vector kernels, FP32-grade arithmetic; integer weights
+//                     as exact integer dot products on the INT8 matrix cores (sp_gemv_i8mfma)
+//   sp_skinny16       5..256 samples, or layers with <= 64 outputs: one operand streamed once through registers
+//                     into 16-bit MFMAs, the thin one in LDS
+//   sp_gemm16_big / sp_gemm16   larger batches: LDS-tiled dequant-to-16-bit MFMA GEMM, fused epilogue
+//   sp_gemm32_f32     FP32 weights beyond 64 samples: FP32 MFMA GEMM
+//   sp_softmax_rows   per-sample softmax (Activation.c:5-21)
+//   sp_eval_*         loss and argmax of a labelled batch (SIMD.c:522-552, Training.c:421-435)
+//   hip_train.inl     the batched training step (included at the end)
 // Weights stay in their serialized form on the device; row-major [out][in]
 // (Private.h:16), element i of an INT4 array in nibble i&1 of byte i/2, element
 // i of an INT2 array at bits 2(i%4) of byte i/4 (Serialize.c:148-152,181-183).
