@@ -98,6 +98,37 @@ def test_forward_leaves_every_layer_in_neurons(S, O):
     S.free_network(net)
 
 
+@pytest.mark.parametrize("fmt,acts", [("i4", ["foo52", "tanh", "softmax"]), ("bf16", ["leaky_relu", "sigmoid", "none"]),
+                                      ("f32", ["relu", "tanh", "softmax"]), ("i2", ["sigmoid", "relu", "none"])])
+def test_repeated_forward_calls_between_other_work_and_reuploads(S, O, fmt, acts):
+    """forward() keeps device buffers, pinned staging and per-layer slots between calls: every one of a series of calls
+    is checked against the oracle, with batched launches on the same stream and a change of the net's arrays in between."""
+    topo = [96, 160, 64, 10]
+    src = make_oracle_net(O, topo, acts, seed=21)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    rng = np.random.default_rng(8)
+    X = rng.standard_normal((12, topo[0])).astype(F32)
+    want = ref.forward_batch(X)
+    for i in range(8):
+        y = S.forward(net, X[i])
+        assert y is not None, S.last_error()
+        assert rel_max_abs(y, want[i]) <= TOL_VEC, (fmt, i)
+        assert np.array_equal(S.neurons_view(net)[:topo[0]], X[i])
+        if i in (3, 5):                                   # launches of another shape in between
+            yb = S.forward_batch(net, X)
+            assert rel_max_abs(yb, want) <= tol_for(fmt, 12)
+    # new weights (FP32 host arrays, packed arrays dropped): the next call must use the re-uploaded arrays
+    for l in range(3):
+        S.weights_view(net, l)[:] = -S.weights_view(net, l)
+        ref.W(l)[:] = -ref.W(l)
+    S.lib().spingalett_hip_invalidate(net)
+    want2 = ref.forward_batch(X)
+    for i in range(5):
+        y = S.forward(net, X[i])
+        assert rel_max_abs(y, want2[i]) <= TOL_VEC, (fmt, "after invalidate", i)
+    S.free_network(net)
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("act", ALL_ACTS)
 def test_every_activation_every_format(S, O, fmt, act):
