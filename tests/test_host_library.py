@@ -287,6 +287,7 @@ def test_reference_header_compiles_against_this_library(S, tmp_path):
     src = tmp_path / "t.c"
     src.write_text(r'''
 #include <Spingalett/Spingalett.h>
+#include <stddef.h>
 #include <stdio.h>
 int main(void) {
     spingalett_set_verbose(false);
@@ -300,6 +301,13 @@ int main(void) {
     free_network(nn);
     NeuralNetwork *l = load_spingalett("abi_model.nn");
     printf("%d %u\n", l != NULL, l ? l->topology[1] : 0u);
+    /* train() links and rejects an empty job the way the reference does (Training.c:609-613) */
+    float x[2] = {0, 1}, t[1] = {1};
+    train(.net = l, .inputs = x, .targets = t, .sample_count = 1, .epochs = 0, .training_strategy = STRATEGY_FULL_BATCH);
+    printf("%d\n", spingalett_last_error_code());
+    spingalett_clear_error();
+    printf("%zu %zu %zu %zu %zu\n", sizeof(TrainArgs), offsetof(TrainArgs, epochs), offsetof(TrainArgs, max_grad_norm),
+           offsetof(TrainArgs, autosave_path), offsetof(TrainArgs, callback_interval));
     free_network(l);
     return spingalett_last_error_code();
 }
@@ -310,4 +318,7 @@ int main(void) {
                            "-Wl,-rpath," + os.path.dirname(S.LIB_PATH)])
     out = subprocess.run([str(exe)], cwd=tmp_path, capture_output=True, text=True)
     assert out.returncode == 0, out
-    assert out.stdout.split() == ["3", "24", "9", "160", "1", "8"]
+    T = S.TrainArgs
+    assert out.stdout.split() == ["3", "24", "9", "160", "1", "8", "2"] + [
+        str(v) for v in (C.sizeof(T), T.epochs.offset, T.max_grad_norm.offset, T.autosave_path.offset,
+                         T.callback_interval.offset)]
