@@ -4,8 +4,8 @@
 //   sp_decode         element decoders (bit-exact with Serialize.c:45-85,195-297)
 //   sp_gemv*          1..4 samples (FP32 weights: up to 64): vector kernels, FP32-grade arithmetic; integer weights
 //                     as exact integer dot products on the INT8 matrix cores (sp_gemv_i8mfma)
-//   sp_skinny16       5..256 samples, or layers with <= 64 outputs: one operand streamed once through registers
-//                     into 16-bit MFMAs, the thin one in LDS
+//   sp_skinny16[_kw]  5..256 samples, or layers with <= 64 outputs: one operand streamed once through registers
+//                     into 16-bit MFMAs, the thin one in LDS (_kw: thin side of <= 8 rows, K split inside the workgroup)
 //   sp_gemm16_big / sp_gemm16   larger batches: LDS-tiled dequant-to-16-bit MFMA GEMM, fused epilogue
 //   sp_gemm32_f32     FP32 weights beyond 64 samples: FP32 MFMA GEMM
 //   sp_softmax_rows   per-sample softmax (Activation.c:5-21)
@@ -1846,6 +1846,207 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
     }
 }
 
+// Variant for a thin operand of at most NCP (8 or 16; the host uses 8) rows: the NW waves of a workgroup share one tile of 32
+// streamed rows and split K among themselves (wave w takes chunks w, w + NW, ...), so that a layer with many streamed
+// rows needs no K split across workgroups, no partial sums in memory and no second launch.  Each wave stages its own
+// thin chunks in its own LDS region (no workgroup barrier in the loop); the NW accumulator tiles meet in LDS at the
+// end and are added in wave order.  Loads and their bookkeeping are those of sp_skinny16.
+template <int FMT, bool F16T, int NCP, int NW>
+__global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
+{
+    using F = SkinnyFmt<FMT>;
+    constexpr int EPL = F::EPL, LPC = F::LPC, BKC = F::BKC, STEPS = F::STEPS, PITCH = F::PITCH;
+    constexpr int UNITS = NCP * (BKC / 16);                // 16-code units of one thin chunk
+    constexpr int UPL = (UNITS + 63) / 64;                 // units per lane
+    constexpr int STAGE = NCP * PITCH;
+    constexpr int NQ = NCP / 2;                            // accumulator registers per lane that belong to thin rows < NCP
+    extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
+
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);   // uniform: chunk addresses stay in scalar registers
+    const uint32_t n31 = lane & 31, h = lane >> 5;
+    const uint32_t K = a.L.K;
+    const uint32_t r_out = blockIdx.x * 32u + n31;
+    const uint32_t kbeg = blockIdx.y * a.kper;
+    const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
+    const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
+    const size_t row_bytes = (size_t)K * F::bits / 8u;
+    uint8_t *my_lds = sk_lds + wave * (2 * STAGE);
+
+    const uint32_t svoff = (uint32_t)((size_t)(r_out < a.R ? r_out : a.R - 1) * row_bytes) + h * 16u;
+    uint32_t tvoff[UPL][2];
+    bool trow_ok[UPL];
+#pragma unroll
+    for (int q = 0; q < UPL; ++q) {
+        const uint32_t u = (uint32_t)lane + 64u * q;
+        const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
+        trow_ok[q] = u < (uint32_t)UNITS && row < a.NC;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) tvoff[q][e] = trow_ok[q] ? (uint32_t)(((size_t)row * K + uc * 16u + 8u * e) * 2u) : 0u;
+    }
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+    // this wave's chunks: w, w + NW, ...; index i of that sequence past the end is clamped to the last one
+    const uint32_t my_n = nchunks > (uint32_t)wave ? (nchunks - (uint32_t)wave + NW - 1) / NW : 0u;
+    const uint32_t last_chunk = nchunks - 1;
+    auto chunk_of = [&](uint32_t i) { return (uint32_t)wave + (i < my_n ? i : my_n - 1) * NW; };
+    constexpr int S_LOADS = LPC, T_LOADS = UPL * 2;
+    auto issue_stream = [&](uint32_t i, u32x4 (&dst)[LPC]) {
+        const uint32_t ch = chunk_of(i);
+        if (ch < last_chunk) {
+            const uint8_t *sb = a.stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
+#pragma unroll
+            for (int j = 0; j < LPC; ++j) {
+                if (j == 0) load16_async<0>(dst[j], svoff, sb);
+                else if (j == 1) load16_async<32>(dst[j], svoff, sb);
+                else if (j == 2) load16_async<64>(dst[j], svoff, sb);
+                else load16_async<96>(dst[j], svoff, sb);
+            }
+        } else {
+            const uint32_t kc0 = kbeg + last_chunk * BKC;
+#pragma unroll
+            for (int j = 0; j < LPC; ++j) {
+                const uint32_t k = kc0 + 2u * j * EPL;                 // first code of the h = 0 lane load
+                const uint32_t add = k + h * EPL < K ? k * F::bits / 8u : 0u - h * 16u;
+                load16_async<0>(dst[j], svoff + add, a.stream);
+            }
+        }
+    };
+    u32x4 thin_regs[UPL][2];
+    auto issue_thin = [&](uint32_t i) {
+        const uint32_t ch = chunk_of(i);
+        if (ch < last_chunk) {
+            const uint16_t *tb = a.thin + (kbeg + ch * BKC);
+#pragma unroll
+            for (int q = 0; q < UPL; ++q)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) load16_async<0>(thin_regs[q][e], tvoff[q][e], tb);
+        } else {
+            const uint32_t kc0 = kbeg + last_chunk * BKC;
+#pragma unroll
+            for (int q = 0; q < UPL; ++q) {
+                const uint32_t uc = ((uint32_t)lane + 64u * q) % (BKC / 16);
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const bool valid = trow_ok[q] && kc0 + uc * 16u + 8u * e + 8u <= kend;
+                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, a.thin);
+                }
+            }
+        }
+    };
+    auto store_thin = [&](int stage, uint32_t i) {
+        const uint32_t kc0 = kbeg + chunk_of(i) * BKC;
+#pragma unroll
+        for (int q = 0; q < UPL; ++q) {
+            const uint32_t u = (uint32_t)lane + 64u * q;
+            if (u >= (uint32_t)UNITS) continue;
+            const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
+            const uint32_t k = kc0 + uc * 16u;
+            const uint32_t keep0 = (trow_ok[q] && k + 8u <= kend) ? 0xFFFFFFFFu : 0u;
+            const uint32_t keep1 = (trow_ok[q] && k + 16u <= kend) ? 0xFFFFFFFFu : 0u;
+            const uint32_t in[8] = {thin_regs[q][0].x & keep0, thin_regs[q][0].y & keep0, thin_regs[q][0].z & keep0,
+                                    thin_regs[q][0].w & keep0, thin_regs[q][1].x & keep1, thin_regs[q][1].y & keep1,
+                                    thin_regs[q][1].z & keep1, thin_regs[q][1].w & keep1};
+            uint32_t o[8];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
+                const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
+                                     ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
+                o[w] = __builtin_amdgcn_perm(in[eb >> 1], in[ea >> 1], sel);
+            }
+            uint8_t *dst = my_lds + stage * STAGE + row * PITCH + uc * 32u;
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+        }
+    };
+    auto compute = [&](int stage, uint32_t i, const u32x4 (&cur)[LPC]) {
+        // lanes of thin rows >= NCP read a row below NCP again: their accumulator rows are never stored
+        const uint8_t *sbase = my_lds + stage * STAGE + (n31 & (NCP - 1)) * PITCH + h * (EPL * 2);
+        const uint32_t kc0 = kbeg + chunk_of(i) * BKC;
+#pragma unroll
+        for (int j = 0; j < LPC; ++j) {
+            const uint32_t keep = (F::bits == 16 && kc0 + (2u * j + h) * EPL >= K) ? 0u : 0xFFFFFFFFu;
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st) {
+                const uint4 tf = *reinterpret_cast<const uint4 *>(sbase + (2 * j * EPL + 8 * st) * 2);
+                uint4 v = make_uint4(cur[j].x, cur[j].y, cur[j].z, cur[j].w);
+                if constexpr (F::bits == 16) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
+                uint32_t sf[4];
+                skinny_frag<FMT>(v, st, sf);
+                if constexpr (F16T) {
+                    f16x8 af, bf;
+                    __builtin_memcpy(&af, &tf, 16);
+                    __builtin_memcpy(&bf, sf, 16);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc, 0, 0, 0);
+                } else {
+                    bf16x8 af, bf;
+                    __builtin_memcpy(&af, &tf, 16);
+                    __builtin_memcpy(&bf, sf, 16);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf, acc, 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto pin_stream = [&](u32x4 (&r)[LPC]) {
+#pragma unroll
+        for (int j = 0; j < LPC; ++j) asm volatile("" : "+v"(r[j]));
+    };
+    auto pin_thin = [&]() {
+#pragma unroll
+        for (int q = 0; q < UPL; ++q)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) asm volatile("" : "+v"(thin_regs[q][e]));
+    };
+    // in flight on entry: streamed chunks i (in `cur`) and i + 1; issued here: thin block i + 1, streamed chunk i + 2
+    auto step = [&](uint32_t i, u32x4 (&cur)[LPC], u32x4 (&far)[LPC]) {
+        const int stage = (int)(i & 1u);
+        issue_thin(i + 1);
+        issue_stream(i + 2, far);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S_LOADS + T_LOADS) : "memory");
+        pin_stream(cur);
+        compute(stage, i, cur);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S_LOADS) : "memory");
+        pin_thin();
+        store_thin(stage ^ 1, i + 1);
+    };
+    if (my_n) {
+        u32x4 ra[LPC], rb[LPC], rc[LPC];
+        issue_thin(0);
+        issue_stream(0, ra);
+        issue_stream(1, rb);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S_LOADS) : "memory");
+        pin_thin();
+        store_thin(0, 0);
+        for (uint32_t i = 0; i < my_n; i += 3) {
+            step(i, ra, rc);
+            if (i + 1 < my_n) step(i + 1, rb, ra);
+            if (i + 2 < my_n) step(i + 2, rc, rb);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the redundant tail loads
+    }
+
+    // accumulator register q of lane (n31, h): thin row 8 (q / 4) + 4 h + q % 4, streamed row n31
+    float *red = reinterpret_cast<float *>(sk_lds + NW * 2 * STAGE);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) red[(wave * NQ + q) * 64 + lane] = acc[q];
+    __syncthreads();
+    if (wave != 0 || r_out >= a.R) return;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        const uint32_t c = 8u * (q >> 2) + 4u * h + (q & 3);
+        if (c >= a.NC) continue;
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[(w * NQ + q) * 64 + lane];
+        if (a.ws) a.ws[((size_t)blockIdx.y * a.NC + c) * a.R + r_out] = sum;
+        else skinny_emit<F16T>(a, c, r_out, sum);
+    }
+}
+
 // adds the K splits of sp_skinny16 and applies bias and activation
 template <bool F16T>
 __global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint32_t splits)
@@ -2327,6 +2528,8 @@ struct ThinCtx {
 struct ThinPlan {
     bool use;
     bool mode_b;
+    bool kw;               // thin operand of <= 8 rows: K split among the waves of a workgroup (sp_skinny16_kw)
+    int ncp;               // thin rows held in LDS in that case
     uint32_t R, NC;        // streamed rows, thin rows
     int rt, ct;
     uint32_t splits, kper, row_blocks, cblocks;
@@ -2350,6 +2553,30 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
         return p;
     }
     const uint32_t bkc = sfmt == I8 ? 128u : (sfmt == I4 || sfmt == I2) ? 256u : 64u;
+    // K split inside the workgroup (sp_skinny16_kw) for thin operands of at most 8 rows.  Every wave then fetches its
+    // own thin chunks (four times the thin traffic, from L2), which pays where the second launch of the split-K path
+    // weighs more: measured faster for INT8 at every size tried, for INT4 / INT2 up to 64 MB and for 16-bit operands
+    // up to 32 MB of streamed bytes, slower beyond (16384 x 16384 INT4 at 8 samples: 40 us against 34 us).
+    const uint64_t streamed_bytes = (uint64_t)p.R * K * (uint64_t)fmt_bits(sfmt) / 8u;
+    const bool kw_pays = sfmt == I8 || streamed_bytes <= ((sfmt == I4 || sfmt == I2) ? (64ull << 20) : (32ull << 20));
+    if (p.NC <= 8u && kw_pays) {
+        // one workgroup per 32 streamed rows, its four waves share K; K is split across workgroups as well only
+        // when the rows alone do not fill the chip
+        p.kw = true;
+        p.ncp = 8;
+        p.rt = p.ct = 1;
+        p.cblocks = 1;
+        p.row_blocks = (p.R + 31u) / 32u;
+        const uint32_t chunks = (K + bkc - 1) / bkc;
+        uint32_t splits = p.row_blocks >= 384u ? 1u : (512u + p.row_blocks - 1) / p.row_blocks;
+        if (splits > 16u) splits = 16u;
+        if (splits > chunks / 4u) splits = chunks / 4u;
+        if (splits < 1u) splits = 1u;
+        const uint32_t cps = (chunks + splits - 1) / splits;
+        p.kper = cps * bkc;
+        p.splits = (chunks + cps - 1) / cps;
+        return p;
+    }
     p.ct = p.NC <= 32 ? 1 : 2;
     p.cblocks = (p.NC + 32u * p.ct - 1) / (32u * p.ct);
     p.rt = (p.R + 255u) / 256u * p.cblocks >= 128u ? 2 : 1;
@@ -2376,11 +2603,24 @@ void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
     kern<<<dim3(p.row_blocks, p.splits, p.cblocks), 256, lds, g_stream>>>(a);
 }
 
+template <int SFMT, bool F16T, int NCP>
+void launch_thin_kw(const SkinnyArgs &a, const ThinPlan &p)
+{
+    constexpr int NW = 4;
+    constexpr size_t lds = (size_t)NW * 2 * NCP * SkinnyFmt<SFMT>::PITCH + (size_t)NW * (NCP / 2) * 64 * sizeof(float);
+    auto kern = sp_skinny16_kw<SFMT, F16T, NCP, NW>;
+    static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+    (void)once;
+    kern<<<dim3(p.row_blocks, p.splits, 1), 64 * NW, lds, g_stream>>>(a);
+}
+
 template <int SFMT, bool F16T>
 void launch_thin(SkinnyArgs a, const ThinPlan &p)
 {
     if (p.splits == 1) a.ws = nullptr;
-    if (p.rt == 2) {
+    if (p.kw) {
+        launch_thin_kw<SFMT, F16T, 8>(a, p);
+    } else if (p.rt == 2) {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 2, 2>(a, p); else launch_thin_inst<SFMT, F16T, 2, 1>(a, p);
     } else {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1>(a, p);
@@ -2398,7 +2638,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
         a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
-        g_last_kernel = "sp_skinny16";
+        g_last_kernel = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
         if (tp.mode_b) {
             a.stream = reinterpret_cast<const uint8_t *>(A);
             a.thin = ctx.w16;

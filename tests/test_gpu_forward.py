@@ -269,6 +269,11 @@ def _decoded_layer(S, fmt, N, K, seed):
     ("i8", 512, 144, 7), ("i8", 2100, 2064, 48), ("i8", 8192, 1024, 200),
     ("i2", 640, 4096, 9), ("i2", 4096, 8192, 64), ("i2", 1000, 320, 130),
     ("bf16", 512, 200, 6), ("bf16", 4096, 2048, 40), ("f16", 1500, 1000, 77), ("f16", 96, 4096, 255),
+    # at most 8 samples (or outputs): K split among the waves of a workgroup (idle waves, K tails, ragged rows), and
+    # the neighbouring sizes that stay on the split-K kernel
+    ("i4", 16384, 2048, 8), ("i4", 300, 4352, 7), ("i8", 12288, 1152, 8), ("i2", 12288, 4096, 6), ("i2", 515, 256, 8),
+    ("bf16", 12300, 584, 8), ("f16", 640, 8200, 5), ("bf16", 96, 64, 5), ("i8", 8, 4096, 1000), ("i2", 3, 2048, 4096),
+    ("i4", 300, 4352, 13), ("i8", 12288, 1152, 16), ("f16", 640, 8200, 12),
     # few outputs, activations streamed
     ("i8", 10, 1000, 256), ("i8", 10, 1000, 4096), ("i4", 64, 512, 1000), ("i2", 33, 2048, 513),
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
