@@ -9,9 +9,9 @@
  * unchanged.  The section "additive interface" lists what this build adds;
  * nothing in the reference interface is altered to make room for it.
  *
- * train() runs its two batched strategies on the device; STRATEGY_SAMPLE and
- * MODE_GENERATOR_FUNCTION are rejected with an error.  Not provided:
- * derivative(), print_parameters().
+ * train() runs on the device (all three strategies; MODE_GENERATOR_FUNCTION is
+ * rejected with an error as in the reference).  Not provided: derivative(),
+ * print_parameters().
  */
 #ifndef SPINGALETT_AMD_H
 #define SPINGALETT_AMD_H
@@ -220,10 +220,13 @@ SPINGALETT_API float activate(float x, ActivationFunction act_func);
  * NULL without an error for a NULL net/input, NULL + ERR_INVALID for fewer
  * than two layers or when no GPU can run it. */
 SPINGALETT_API float *forward_struct_arguments(ForwardArgs args);
-/* Spingalett.h:229-230 (Training.c:584-949).  STRATEGY_FULL_BATCH and STRATEGY_SMALL_BATCH run every
- * step on the device in FP32 (forward keeping all layers, deltas, gradients scaled by 1/batch,
- * optional clipping by the global norm, SGD / momentum / RMSprop / Adam / AdamW update), with the
- * reference's epoch loop around them: shuffle per epoch, loss report, NaN check, autosave, callback.
+/* Spingalett.h:229-230 (Training.c:584-949).  Every step runs on the device in FP32 (forward keeping all
+ * layers, deltas, gradients scaled by 1/batch, optional clipping by the global norm, SGD / momentum /
+ * RMSprop / Adam / AdamW update), with the reference's epoch loop around them: shuffle per epoch
+ * (mini-batches), loss report, NaN check, autosave, callback.  STRATEGY_SAMPLE (the zero value) applies one
+ * update per sample in the given order with the rules of backpropagation() (Training.c:78-213: no
+ * clipping, RMSprop folds the decay into the gradient); it costs one small device step per sample, so the
+ * two batched strategies are the ones to use for speed.
  * The host arrays (weights, biases, gradients, moments) are current whenever the callback, the NaN
  * check or autosave look at them and when the call returns; time_step advances once per step.
  * A net loaded from a quantized file is trained from its FP32 host arrays (what the reference's

@@ -108,6 +108,9 @@ typedef struct {
     float learning_rate, weight_decay, momentum, beta1, beta2, epsilon;
     float max_grad_norm;    /* > 0: gradients are scaled to this global L2 norm when they exceed it */
     float beta1_pow_t, beta2_pow_t;   /* beta^t of the step being applied (Training.c:743-745) */
+    int32_t decay_in_grad;  /* RMSprop only.  0: the batched rule, W -= lr (decay W + g / sqrt(v + eps)) with v from g
+                               (SIMD.c:455-494); 1: the per-sample rule of backpropagation(), decay W joins g before
+                               v is updated (Training.c:196-211) */
 } sphip_train_args;
 
 /* arrays of sphip_train_set / sphip_train_get; layer l = 0 .. layers-2, weights row-major [out][in] */

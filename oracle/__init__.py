@@ -45,7 +45,7 @@ _lib = None
 class _OptArgs(C.Structure):
     _fields_ = [("optimizer", C.c_int), ("learning_rate", C.c_float), ("weight_decay", C.c_float),
                 ("momentum", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("epsilon", C.c_float),
-                ("max_grad_norm", C.c_float)]
+                ("max_grad_norm", C.c_float), ("decay_in_grad", C.c_int)]
 
 
 OPT_SGD, OPT_MOMENTUM, OPT_RMSPROP, OPT_ADAM, OPT_ADAMW = range(5)
@@ -234,11 +234,12 @@ class Net:
 
     def apply_gradients(self, state: "TrainState", gW: np.ndarray, gB: np.ndarray, optimizer: int,
                         lr: float = 0.01, weight_decay: float = 0.0, momentum: float = 0.9, beta1: float = 0.9,
-                        beta2: float = 0.999, epsilon: float = 1e-8, max_grad_norm: float = 0.0) -> None:
+                        beta2: float = 0.999, epsilon: float = 1e-8, max_grad_norm: float = 0.0,
+                        decay_in_grad: bool = False) -> None:
         """One optimizer step in place (weights, biases, state; gW / gB are modified like the reference's)."""
         state.beta1_pow *= np.float32(beta1)
         state.beta2_pow *= np.float32(beta2)
-        a = _OptArgs(optimizer, lr, weight_decay, momentum, beta1, beta2, epsilon, max_grad_norm)
+        a = _OptArgs(optimizer, lr, weight_decay, momentum, beta1, beta2, epsilon, max_grad_norm, int(decay_in_grad))
         lib().orc_apply_gradients(self._h, C.byref(a), _ptr(gW), _ptr(gB), _ptr(state.mW), _ptr(state.vW),
                                   _ptr(state.mB), _ptr(state.vB), float(state.beta1_pow), float(state.beta2_pow))
 

@@ -711,6 +711,13 @@ static void opt_update(const orc_opt_args *a, float *W, float *g, float *m, floa
     }
     case ORC_OPT_RMSPROP:                                             /* :455-494 */
         for (uint64_t i = 0; i < cnt; ++i) {
+            if (a->decay_in_grad) {                                   /* backpropagation(), Training.c:196-211 */
+                float grad = g[i];
+                if (decay > 0.0f) grad += decay * W[i];
+                v[i] = b2 * v[i] + omb2 * (grad * grad);
+                W[i] -= lr * grad / sqrtf(v[i] + eps);
+                continue;
+            }
             v[i] = b2 * v[i] + omb2 * (g[i] * g[i]);
             const float v_hat = v[i] + eps;
             W[i] -= lr * (decay * W[i] + g[i] / sqrtf(v_hat));

@@ -133,6 +133,7 @@ enum { ORC_OPT_SGD = 0, ORC_OPT_MOMENTUM, ORC_OPT_RMSPROP, ORC_OPT_ADAM, ORC_OPT
 typedef struct {
     int   optimizer;
     float learning_rate, weight_decay, momentum, beta1, beta2, epsilon, max_grad_norm;
+    int   decay_in_grad;   /* RMSprop: 1 = the per-sample rule of backpropagation() (Training.c:196-211) */
 } orc_opt_args;
 /* derivative of an activation as a function of its output (Activation.c:40-56) */
 float orc_derivative(float a, int act);

@@ -110,7 +110,7 @@ class SphipTrainArgs(C.Structure):
     _fields_ = [("optimizer", C.c_int32), ("loss_func", C.c_int32), ("learning_rate", C.c_float),
                 ("weight_decay", C.c_float), ("momentum", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float),
                 ("epsilon", C.c_float), ("max_grad_norm", C.c_float), ("beta1_pow_t", C.c_float),
-                ("beta2_pow_t", C.c_float)]
+                ("beta2_pow_t", C.c_float), ("decay_in_grad", C.c_int32)]
 
 
 class SphipDesc(C.Structure):

@@ -320,13 +320,7 @@ void train_struct_arguments(TrainArgs args)
         sp_log(LOG_ERROR, "Invalid training arguments");
         return;
     }
-    if (args.training_strategy == STRATEGY_SAMPLE) {
-        /* the reference's per-sample loop (Training.c:78-213) is a sequence of single-sample updates;
-         * the device back-end provides the two batched strategies only */
-        sp_set_error(SPINGALETT_ERR_INVALID, "HIP back-end: STRATEGY_SAMPLE is not provided; use STRATEGY_SMALL_BATCH or STRATEGY_FULL_BATCH");
-        sp_log(LOG_ERROR, "HIP back-end: STRATEGY_SAMPLE is not provided; use STRATEGY_SMALL_BATCH or STRATEGY_FULL_BATCH");
-        return;
-    }
+    const bool per_sample = args.training_strategy == STRATEGY_SAMPLE;
     const bool small = args.training_strategy == STRATEGY_SMALL_BATCH;
     if (small && args.batch_size == 0) args.batch_size = 32;
     if (small && args.batch_size > sample_count) args.batch_size = sample_count;
@@ -360,6 +354,8 @@ void train_struct_arguments(TrainArgs args)
         }
     }
 
+    if (per_sample)
+        sp_log(LOG_WARNING, "HIP back-end: the per-sample strategy runs one small device step per sample; the batched strategies are the fast ones");
     if (small)
         sp_log(LOG_INFO, "Starting training: loss=%s, strategy=%s, mode=ARRAY, optimizer=%s, compute=HIP, batch_size=%u",
                sp_loss_names[net->loss_func], strategy_names[args.training_strategy], optimizer_names[args.optimizer_type], args.batch_size);
@@ -368,7 +364,7 @@ void train_struct_arguments(TrainArgs args)
                sp_loss_names[net->loss_func], strategy_names[args.training_strategy], optimizer_names[args.optimizer_type]);
 
     const uint32_t in_sz = net->topology[0], out_sz = net->topology[net->layers - 1];
-    const uint32_t eff_batch = small ? args.batch_size : sample_count;
+    const uint32_t eff_batch = small ? args.batch_size : per_sample ? 1u : sample_count;
     uint32_t *order = NULL;
     float *bx = NULL, *bt = NULL;
     if (small) {
@@ -391,12 +387,28 @@ void train_struct_arguments(TrainArgs args)
         .beta1 = args.beta1, .beta2 = args.beta2, .epsilon = args.epsilon, .max_grad_norm = args.max_grad_norm,
         .beta1_pow_t = 1.0f, .beta2_pow_t = 1.0f,                                   /* Training.c:684-685 */
     };
+    if (per_sample) {
+        /* backpropagation() (Training.c:78-213): one update per sample in the given order, no clipping,
+         * RMSprop folds the decay into the gradient */
+        ta.max_grad_norm = 0.0f;
+        ta.decay_in_grad = 1;
+    }
     bool failed = false;
     for (size_t epoch = 1; epoch <= epochs && !failed; ++epoch) {
         const bool need_loss = should_report(epoch, epochs, args.report_interval) ||
                                (args.callback && should_report(epoch, epochs, args.callback_interval));
         float total_error = 0.0f;
-        if (!small) {
+        if (per_sample) {
+            for (uint32_t s = 0; s < sample_count && !failed; ++s) {
+                float loss = 0.0f;
+                net->time_step++;
+                ta.beta1_pow_t *= args.beta1;
+                ta.beta2_pow_t *= args.beta2;
+                failed = sphip_train_step(sn->dev, args.inputs + (size_t)s * in_sz, args.targets + (size_t)s * out_sz, 1, &ta, 0,
+                                          need_loss ? &loss : NULL) != 0;
+                total_error += loss;
+            }
+        } else if (!small) {
             float loss = 0.0f;
             net->time_step++;
             ta.beta1_pow_t *= args.beta1;

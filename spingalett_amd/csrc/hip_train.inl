@@ -261,6 +261,7 @@ struct OptArgs {
     uint64_t cnt;
     const float *clip;     // device scalar the gradient is multiplied by first, or nullptr
     int opt;               // OptimizerType, Spingalett.h:76-83
+    int decay_in_grad;     // RMSprop: decay * W joins the gradient before the second moment (per-sample rule)
     float lr, decay, momentum, b1, b2, omb1, omb2, mf, vf, eps;
 };
 
@@ -284,9 +285,10 @@ __global__ __launch_bounds__(256) void sp_train_opt(const OptArgs a)
         break;
     }
     case 2: {   // RMSprop
+        if (a.decay_in_grad && a.decay > 0.0f) g += a.decay * w;
         const float v = a.b2 * a.v[i] + a.omb2 * (g * g);
         a.v[i] = v;
-        w -= a.lr * (a.decay * w + g / sqrtf(v + a.eps));
+        w -= a.decay_in_grad ? a.lr * g / sqrtf(v + a.eps) : a.lr * (a.decay * w + g / sqrtf(v + a.eps));
         break;
     }
     default: {  // Adam (3): decay joins the gradient; AdamW (4): decay shrinks the weight
@@ -403,6 +405,7 @@ void launch_opt(const sphip_train_args &a, float *W, float *g, float *m, float *
     OptArgs o{};
     o.W = W; o.g = g; o.m = m; o.v = v; o.cnt = cnt; o.clip = clip;
     o.opt = a.optimizer;
+    o.decay_in_grad = a.decay_in_grad;
     o.lr = a.learning_rate; o.decay = decay; o.momentum = a.momentum;
     o.b1 = a.beta1; o.b2 = a.beta2;
     // formed in FP32 like the reference's locals (Training.c:447-448, 479-480)

@@ -246,6 +246,63 @@ def test_callback_stops_training_and_autosave_writes_files(tmp_path):
     S.free_network(net)
 
 
+@pytest.mark.parametrize("opt,kw", [(S.OPTIMIZER_SGD, {"weight_decay": 0.1}), (S.OPTIMIZER_MOMENTUM, {}),
+                                    (S.OPTIMIZER_RMSPROP, {"weight_decay": 0.2}), (S.OPTIMIZER_ADAM, {}),
+                                    (S.OPTIMIZER_ADAMW, {"weight_decay": 0.1})])
+def test_per_sample_strategy_matches_oracle(opt, kw):
+    """STRATEGY_SAMPLE: one update per sample in order with the rules of backpropagation() (Training.c:78-213);
+    max_grad_norm is not applied there."""
+    topo, acts, loss, n, epochs = [6, 12, 4], ["tanh", "softmax"], 1, 9, 2
+    net, onet = public_net(topo, acts, loss, seed=13)
+    rng = np.random.default_rng(4)
+    X = rng.standard_normal((n, topo[0])).astype(np.float32)
+    T = targets_for(rng, n, topo[-1], True)
+    errs = []
+    S.clear_error()
+    S.train(net, X, T, epochs, S.STRATEGY_SAMPLE, opt, learning_rate=0.02, max_grad_norm=1e-3,
+            callback=lambda p, epoch, err: errs.append(err) or False, **kw)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    st = O.TrainState(onet)
+    want = []
+    for _ in range(epochs):
+        total = 0.0
+        for s_ in range(n):
+            gW, gB, out = onet.batch_gradients(X[s_:s_ + 1], T[s_:s_ + 1], grad_scale=1.0)
+            total += O.batch_loss(out, T[s_:s_ + 1], loss, O.ACT["softmax"])
+            onet.apply_gradients(st, gW, gB, opt, lr=0.02, decay_in_grad=True, **kw)
+        want.append(total / n)
+    for l in range(len(topo) - 1):
+        assert rel_max_abs(S.weights_view(net, l), onet.W(l)) <= TOL, l
+        assert rel_max_abs(S.biases_view(net, l), onet.b(l)) <= TOL, l
+    assert errs == pytest.approx(want, rel=1e-4)
+    assert net.contents.time_step == epochs * n
+    S.free_network(net)
+
+
+def test_xor_with_the_example_settings_converges():
+    """The reference's end-to-end sanity check (Examples/XOR.c:27-64): 2-8-1, FOO52 / sigmoid, He / Xavier start, squared
+    error, full batch, AdamW 0.01 with decay 1e-4, 10,000 epochs; every output within 0.1 of its target."""
+    X = np.float32([[0, 0], [0, 1], [1, 0], [1, 1]])
+    T = np.float32([[0], [1], [1], [0]])
+    passed = 0
+    for attempt in range(3):                                   # the start is random, as in the example
+        net = S.new_spingalett(S.LOSS_MSE)
+        S.layer(net, 2)
+        S.layer(net, 8, S.ACT_FOO52, S.WEIGHT_INITIALIZATION_HE)
+        S.layer(net, 1, S.ACT_SIGMOID, S.WEIGHT_INITIALIZATION_XAVIER)
+        reports = []
+        S.clear_error()
+        S.train(net, X, T, 10000, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAMW, learning_rate=0.01, weight_decay=1e-4,
+                callback=lambda p, epoch, err: reports.append(epoch) or False, callback_interval=5000)
+        assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+        assert reports == [5000, 10000]
+        passed = sum(abs(float(S.forward(net, X[i])[0]) - float(T[i, 0])) < 0.1 for i in range(4))
+        S.free_network(net)
+        if passed == 4:
+            break
+    assert passed == 4
+
+
 def test_train_rejects_what_the_reference_rejects():
     net, _ = public_net([4, 6, 2], ["softmax", "none"], 0)
     X, T = np.zeros((3, 4), np.float32), np.zeros((3, 2), np.float32)
@@ -257,7 +314,7 @@ def test_train_rejects_what_the_reference_rejects():
     w0 = S.weights_view(net, 0).copy()
     for kw, msg in (({"training_mode": S.MODE_GENERATOR_FUNCTION}, "Generator function"),
                     ({"sample_count": 0}, "Invalid training arguments"),
-                    ({"strategy": S.STRATEGY_SAMPLE}, "STRATEGY_SAMPLE")):
+                    ({"strategy": 7}, "unknown optimizer, strategy or loss")):
         S.clear_error()
         S.train(net, X, T, 1, **kw)
         code, text = S.last_error()

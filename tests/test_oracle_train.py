@@ -222,6 +222,27 @@ def test_rmsprop_first_step():
     assert not st.mW.any()                                    # no first moment
 
 
+def test_rmsprop_per_sample_rule_folds_decay_into_the_gradient():
+    """backpropagation() (Training.c:196-211): decay * W joins the gradient before the second moment."""
+    lr, b2, eps, wd = 0.02, 0.9, 1e-6, 0.4
+    net, st, gW, gB = _fresh()
+    w0, b0 = net.weights.copy(), net.biases.copy()
+    net.apply_gradients(st, gW.copy(), gB.copy(), O.OPT_RMSPROP, lr=lr, beta2=b2, epsilon=eps, weight_decay=wd,
+                        decay_in_grad=True)
+    omb2 = float(np.float32(1) - np.float32(b2))
+    g = gW.astype(np.float64) + wd * w0
+    np.testing.assert_allclose(net.weights, w0 - lr * g / np.sqrt(omb2 * g ** 2 + eps), rtol=2e-5, atol=1e-7)
+    np.testing.assert_allclose(st.vW, omb2 * g ** 2, rtol=1e-5)
+    gb = gB.astype(np.float64)                                # biases carry no decay in either rule
+    np.testing.assert_allclose(net.biases, b0 - lr * gb / np.sqrt(omb2 * gb ** 2 + eps), rtol=2e-5, atol=1e-7)
+    # without decay the two rules coincide up to the rounding of lr * g / sqrt(.) against lr * (g / sqrt(.))
+    n1, s1, g1, h1 = _fresh()
+    n2, s2, g2, h2 = _fresh()
+    n1.apply_gradients(s1, g1, h1, O.OPT_RMSPROP, lr=lr, beta2=b2, epsilon=eps)
+    n2.apply_gradients(s2, g2, h2, O.OPT_RMSPROP, lr=lr, beta2=b2, epsilon=eps, decay_in_grad=True)
+    np.testing.assert_allclose(n1.weights, n2.weights, rtol=1e-6)
+
+
 def test_clipping_precedes_the_update():
     net, st, gW, gB = _fresh()
     w0 = net.weights.copy()
