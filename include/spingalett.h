@@ -10,8 +10,7 @@
  * nothing in the reference interface is altered to make room for it.
  *
  * train() runs on the device (all three strategies; MODE_GENERATOR_FUNCTION is
- * rejected with an error as in the reference).  Not provided: derivative(),
- * print_parameters().
+ * rejected with an error as in the reference).
  */
 #ifndef SPINGALETT_AMD_H
 #define SPINGALETT_AMD_H
@@ -215,6 +214,8 @@ SPINGALETT_API NeuralNetwork *new_spingalett_struct_arguments(NeuralNetworkArgs 
 SPINGALETT_API void layer_struct_arguments(LayerArgs args);
 /* Spingalett.h:223 (Activation.c:23-38) */
 SPINGALETT_API float activate(float x, ActivationFunction act_func);
+/* Spingalett.h:224 (Activation.c:40-56): slope of the activation as a function of its output. */
+SPINGALETT_API float derivative(float x, ActivationFunction act_func);
 /* Spingalett.h:226-227 (Network.c:202-251): one sample.  Returns a pointer
  * into net->neurons (last layer), valid until the next call on that net;
  * NULL without an error for a NULL net/input, NULL + ERR_INVALID for fewer
@@ -238,6 +239,8 @@ SPINGALETT_API void save_spingalett_struct_arguments(SaveArgs args);
  * reference; additionally keeps the packed arrays so the device receives the
  * serialized bytes, not the FP32 expansion. */
 SPINGALETT_API NeuralNetwork *load_spingalett(const char *filename);
+/* Spingalett.h:237 (Network.c:253-281): loss, activations, every bias and weight of the host arrays as LOG_INFO lines. */
+SPINGALETT_API void print_parameters(NeuralNetwork *net);
 /* Spingalett.h:238 (Network.c:283-301); also releases device memory. */
 SPINGALETT_API void free_network(NeuralNetwork *net);
 

@@ -131,7 +131,7 @@ PUBLIC_SYMBOLS = [
     "spingalett_set_dequant_mode", "spingalett_get_dequant_mode", "spingalett_forward_batch",
     "spingalett_forward_batch_device", "spingalett_hip_synchronize", "spingalett_hip_invalidate",
     "spingalett_hip_precision", "spingalett_hip_decode", "spingalett_hip_handle", "load_spingalett_memory",
-    "spingalett_evaluate_batch", "train_struct_arguments",
+    "spingalett_evaluate_batch", "train_struct_arguments", "derivative", "print_parameters",
 ]
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
@@ -196,6 +196,8 @@ def lib():
                                             C.c_void_p, C.POINTER(C.c_uint32)]
     L.spingalett_evaluate_batch.restype = C.c_int
     L.train_struct_arguments.argtypes = [TrainArgs]; L.train_struct_arguments.restype = None
+    L.derivative.argtypes = [C.c_float, C.c_int]; L.derivative.restype = C.c_float
+    L.print_parameters.argtypes = [NetPtr]; L.print_parameters.restype = None
     L.spingalett_hip_synchronize.restype = C.c_int
     L.spingalett_hip_invalidate.argtypes = [NetPtr]; L.spingalett_hip_invalidate.restype = None
     L.spingalett_hip_precision.argtypes = [NetPtr]; L.spingalett_hip_precision.restype = C.c_int
@@ -360,6 +362,14 @@ def load_spingalett_memory(data: bytes):
 
 def free_network(net):
     lib().free_network(net)
+
+
+def derivative(x: float, act: int) -> float:
+    return float(lib().derivative(x, act))
+
+
+def print_parameters(net):
+    lib().print_parameters(net)
 
 
 def activate(x: float, act: int) -> float:

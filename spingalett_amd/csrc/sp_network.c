@@ -76,6 +76,42 @@ float activate(float x, ActivationFunction act)
     }
 }
 
+/* ---- derivative (Activation.c:40-56): slope of an activation as a function of its OUTPUT ---- */
+float derivative(float x, ActivationFunction act)
+{
+    switch (act) {
+    case ACT_RELU:       return x > 0.0f ? 1.0f : 0.0f;
+    case ACT_LEAKY_RELU: return x > 0.0f ? 1.0f : 0.01f;
+    case ACT_SIGMOID:
+    case ACT_SOFTMAX:    return x * (1.0f - x);
+    case ACT_TANH:       return 1.0f - x * x;
+    case ACT_FOO52:      return (x > 1.0f || x < 0.0f) ? 0.01f : 1.0f;
+    default:             return 1.0f;
+    }
+}
+
+/* ---- print_parameters (Network.c:253-281): every bias and weight of the host arrays through the log ---- */
+void print_parameters(NeuralNetwork *net)
+{
+    if (!net) return;
+    sp_log(LOG_INFO, "========== DEBUG NETWORK PARAMETERS ==========");
+    sp_log(LOG_INFO, "Loss Function: %s", sp_loss_names[net->loss_func]);
+    for (uint32_t l = 0; l + 1 < net->layers; ++l) {
+        const uint32_t in = net->topology[l], out = net->topology[l + 1];
+        sp_log(LOG_INFO, "[Connection: Layer %u (%u neurons) -> Layer %u (%u neurons), activation function: %s]",
+               l, in, l + 1, out, sp_act_names[net->act_func[l]]);
+        sp_log(LOG_INFO, "  Biases (Thresholds) for Layer %u:", l + 1);
+        for (uint32_t k = 0; k < out; ++k)
+            sp_log(LOG_INFO, "    Neuron %u bias: %12.6g", k, (double)net->biases[net->bias_offsets[l] + k]);
+        sp_log(LOG_INFO, "  Weights: (total: %llu)", (unsigned long long)((uint64_t)in * out));
+        for (uint32_t k = 0; k < in; ++k)
+            for (uint32_t j = 0; j < out; ++j)
+                sp_log(LOG_INFO, "    L%u N%u -> L%u N%u: %12.6g", l, k, l + 1, j,
+                       (double)net->weights[net->weight_offsets[l] + (uint64_t)j * in + k]);
+    }
+    sp_log(LOG_INFO, "================================================");
+}
+
 /* ---- new_spingalett (Network.c:34-45) ---- */
 NeuralNetwork *new_spingalett_struct_arguments(NeuralNetworkArgs args)
 {

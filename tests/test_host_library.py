@@ -236,6 +236,43 @@ def test_activate_matches_oracle(S, O):
         assert np.allclose(got, want, rtol=2e-7, atol=0), a
 
 
+def test_derivative_matches_oracle(S, O):
+    xs = np.array([-0.5, 0.0, 0.25, 1.0, 1.5], np.float32)
+    for a in range(7):
+        got = np.array([S.derivative(float(x), a) for x in xs], np.float32)
+        assert np.array_equal(got, O.derivative(xs, a)), a
+
+
+def test_print_parameters_lists_every_bias_and_weight(S):
+    """print_parameters (Network.c:253-281) goes through the log: one line per bias and per weight, weights listed input
+    neuron by input neuron."""
+    lines = []
+    cb = C.CFUNCTYPE(None, C.c_int, C.c_char_p)(lambda level, msg: lines.append((level, msg.decode())))
+    net = S.new_spingalett(S.LOSS_CROSS_ENTROPY)
+    S.layer(net, 2)
+    S.layer(net, 3, S.ACT_TANH, S.WEIGHT_INITIALIZATION_NONE)
+    S.weights_view(net, 0)[:] = np.arange(6, dtype=np.float32).reshape(3, 2) + 1       # W[j][k] = 1 + 2 j + k
+    S.biases_view(net, 0)[:] = [0.5, -0.5, 0.25]
+    S.lib().spingalett_set_log_callback(cb)
+    S.lib().spingalett_set_log_level(S.LOG_INFO)
+    S.set_verbose(True)
+    try:
+        S.print_parameters(net)
+    finally:
+        S.set_verbose(False)
+        S.lib().spingalett_set_log_callback(C.CFUNCTYPE(None, C.c_int, C.c_char_p)())
+    text = [m for lvl, m in lines if lvl == S.LOG_INFO]
+    assert any("Cross-Entropy" in m for m in text)
+    assert any("Layer 0 (2 neurons) -> Layer 1 (3 neurons)" in m and "Tanh" in m for m in text)
+    assert sum("bias:" in m for m in text) == 3
+    weights = [m for m in text if "->" in m and m.lstrip().startswith("L0 N")]
+    assert len(weights) == 6
+    assert weights[0].split(":")[0].strip() == "L0 N0 -> L1 N0" and float(weights[0].split(":")[1]) == 1.0
+    assert weights[1].split(":")[0].strip() == "L0 N0 -> L1 N1" and float(weights[1].split(":")[1]) == 3.0
+    assert weights[3].split(":")[0].strip() == "L0 N1 -> L1 N0" and float(weights[3].split(":")[1]) == 2.0
+    S.free_network(net)
+
+
 def test_settings_and_error_slot(S):
     L = S.lib()
     assert L.spingalett_get_compute_mode() == S.COMPUTE_HIP
