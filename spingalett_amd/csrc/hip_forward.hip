@@ -1548,6 +1548,19 @@ __host__ __device__ constexpr int skinny_perm(int p)
     return p;
 }
 
+// the 16 codes of a unit of the thin operand (eight 16-bit pairs) in the order skinny_perm gives
+template <int FMT>
+__device__ __forceinline__ void skinny_permute_unit(const uint32_t (&in)[8], uint32_t (&o)[8])
+{
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
+        const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
+                             ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
+        o[w] = __builtin_amdgcn_perm(in[eb >> 1], in[ea >> 1], sel);
+    }
+}
+
 typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t magic_sub(uint32_t v, uint32_t c)
@@ -1748,13 +1761,7 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
                                     thin_regs[q][0].w & keep0, thin_regs[q][1].x & keep1, thin_regs[q][1].y & keep1,
                                     thin_regs[q][1].z & keep1, thin_regs[q][1].w & keep1};
             uint32_t o[8];
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
-                const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
-                                     ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
-                o[w] = __builtin_amdgcn_perm(in[eb >> 1], in[ea >> 1], sel);
-            }
+            skinny_permute_unit<FMT>(in, o);
             uint8_t *dst = sk_lds + stage * STAGE + row * PITCH + uc * 32u;
             *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
             *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(o[4], o[5], o[6], o[7]);
@@ -1951,13 +1958,7 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
                                     thin_regs[q][0].w & keep0, thin_regs[q][1].x & keep1, thin_regs[q][1].y & keep1,
                                     thin_regs[q][1].z & keep1, thin_regs[q][1].w & keep1};
             uint32_t o[8];
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                const int ea = skinny_perm<FMT>(2 * w), eb = skinny_perm<FMT>(2 * w + 1);
-                const uint32_t sel = (uint32_t)(2 * (ea & 1)) | ((uint32_t)(2 * (ea & 1) + 1) << 8) |
-                                     ((uint32_t)(4 + 2 * (eb & 1)) << 16) | ((uint32_t)(4 + 2 * (eb & 1) + 1) << 24);
-                o[w] = __builtin_amdgcn_perm(in[eb >> 1], in[ea >> 1], sel);
-            }
+            skinny_permute_unit<FMT>(in, o);
             uint8_t *dst = my_lds + stage * STAGE + row * PITCH + uc * 32u;
             *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
             *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(o[4], o[5], o[6], o[7]);

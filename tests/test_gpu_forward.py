@@ -274,6 +274,7 @@ def _decoded_layer(S, fmt, N, K, seed):
     ("i4", 16384, 2048, 8), ("i4", 300, 4352, 7), ("i8", 12288, 1152, 8), ("i2", 12288, 4096, 6), ("i2", 515, 256, 8),
     ("bf16", 12300, 584, 8), ("f16", 640, 8200, 5), ("bf16", 96, 64, 5), ("i8", 8, 4096, 1000), ("i2", 3, 2048, 4096),
     ("i4", 300, 4352, 13), ("i8", 12288, 1152, 16), ("f16", 640, 8200, 12),
+    ("i8", 1, 64, 100), ("f16", 2, 8, 9), ("i2", 4, 16, 5),             # one to four outputs, K below one chunk
     # few outputs, activations streamed
     ("i8", 10, 1000, 256), ("i8", 10, 1000, 4096), ("i4", 64, 512, 1000), ("i2", 33, 2048, 513),
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
