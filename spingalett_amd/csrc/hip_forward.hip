@@ -1523,6 +1523,7 @@ struct SkinnyArgs {
     void *C;                 // [M][N]
     float *ws;               // [S][NC][R] partial sums when the grid splits K
     uint32_t R, NC;          // streamed rows, thin rows
+    uint32_t row_blocks, cblocks;   // workgroups along the streamed rows / blocks of thin rows (grid x covers both)
     uint32_t kper;           // codes per K split (whole chunks)
     int out_f32;
     int mode_b;              // 0: streamed rows are outputs, thin rows samples; 1: the reverse
@@ -1650,8 +1651,18 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint32_t n31 = lane & 31, h = lane >> 5;
     const uint32_t K = a.L.K;
-    const uint32_t row0 = (blockIdx.x * 4u + (uint32_t)wave) * (32u * RT);
-    const uint32_t cbase = blockIdx.z * (32u * CT);
+    // Grid x enumerates (row block, thin block).  Consecutive workgroup ids go to consecutive dies (eight of them,
+    // each with its own L2): the thin blocks of one row block get ids eight apart, so they run on the same die at
+    // about the same time and the second and later ones find the streamed rows in its L2.
+    uint32_t rblk = blockIdx.x, cblk = 0;
+    if (a.cblocks > 1) {
+        const uint32_t per = 8u * a.cblocks, group = blockIdx.x / per, rem = blockIdx.x % per;
+        rblk = group * 8u + (rem & 7u);
+        cblk = rem >> 3;
+        if (rblk >= a.row_blocks) return;                 // padding of the last group
+    }
+    const uint32_t row0 = (rblk * 4u + (uint32_t)wave) * (32u * RT);
+    const uint32_t cbase = cblk * (32u * CT);
     const uint32_t kbeg = blockIdx.y * a.kper;
     const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
     const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
@@ -2536,13 +2547,26 @@ struct ThinPlan {
     uint32_t splits, kper, row_blocks, cblocks;
 };
 
+// Largest batch the weight-streaming kernel takes before the tiled GEMM does better (which runs from 65 samples up, a
+// partly filled row of 256 x 256 tiles).  Measured on whole nets: 8192-wide BF16 layers 417 / 439 / 475 us at 72 / 96 /
+// 128 samples through the GEMM against 468 / 486 / 502 us streaming (and 576 against 918 us at 256); 16384-wide INT4
+// 281 / 305 us at 192 / 256 against 366 / 369 us, but 257 / 263 us at 96 / 128 against 213 / 233 us; 8192-wide INT2 still
+// 8 % better streaming at 256.  The fewer bytes a code has, the longer re-reading the weights per block of 64 samples pays.
+// Layers of a few megabytes stay with the streaming kernel up to 256 samples (the 784-512-1000-10 INT8 net: 36 us
+// against 57 us at 256 samples).
+uint32_t thin_max_samples(int fmt, uint32_t N, uint32_t K)
+{
+    if ((uint64_t)N * K * (uint64_t)fmt_bits(fmt) / 8u <= (8ull << 20)) return 256u;
+    return fmt_bits(fmt) == 16 ? 64u : fmt == I2 ? 256u : 128u;
+}
+
 // mode_b streams 16-bit activations (fmt = the activation type), mode a the weights
 ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
 {
     ThinPlan p{};
     if (N <= 64 && K % 8u == 0 && M >= 1) {
         p.use = true; p.mode_b = true; p.R = M; p.NC = N;
-    } else if (M <= 256 && rows_aligned(fmt, K) && K % 8u == 0) {
+    } else if (M <= thin_max_samples(fmt, N, K) && rows_aligned(fmt, K) && K % 8u == 0) {
         p.use = true; p.mode_b = false; p.R = N; p.NC = M;
     } else {
         return p;
@@ -2601,7 +2625,8 @@ void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
     auto kern = sp_skinny16<SFMT, F16T, RT, CT>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
     (void)once;
-    kern<<<dim3(p.row_blocks, p.splits, p.cblocks), 256, lds, g_stream>>>(a);
+    const uint32_t gx = p.cblocks > 1 ? (p.row_blocks + 7u) / 8u * 8u * p.cblocks : p.row_blocks;
+    kern<<<dim3(gx, p.splits, 1), 256, lds, g_stream>>>(a);
 }
 
 template <int SFMT, bool F16T, int NCP>
@@ -2638,7 +2663,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const ThinPlan tp = plan_thin(FMT, M, L.N, L.K);
     if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
-        a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
+        a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.row_blocks = tp.row_blocks; a.cblocks = tp.cblocks; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
         g_last_kernel = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
         if (tp.mode_b) {
             a.stream = reinterpret_cast<const uint8_t *>(A);
@@ -2658,7 +2683,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const uint32_t big_tiles = ((M + 255u) / 256u) * ((L.N + 255u) / 256u);
     const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
-    if (aligned && L.K % 64u == 0 && M >= 256 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
+    if (aligned && L.K % 64u == 0 && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
         constexpr int BM = 256, BN = 256;
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
         else g.ws = ctx.ws;
