@@ -2684,16 +2684,24 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
     if (aligned && L.K % 64u == 0 && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
-        constexpr int BM = 256, BN = 256;
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
         else g.ws = ctx.ws;
         const dim3 grid(big_tiles, g.ws ? splits : 1u);
-        constexpr size_t lds = 2 * (BM + BN) * 64 * sizeof(uint16_t);
         g_last_kernel = "sp_gemm16_big";
-        auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
-        static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-        (void)once;
-        kern<<<grid, 512, lds, g_stream>>>(g);
+        if (M <= 128u) {
+            // a single row of tiles: 128 rows instead of 256 half-empty ones
+            constexpr size_t lds = 2 * (128 + 256) * 64 * sizeof(uint16_t);
+            auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 2, 2>;
+            static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            kern<<<grid, 512, lds, g_stream>>>(g);
+        } else {
+            constexpr size_t lds = 2 * (256 + 256) * 64 * sizeof(uint16_t);
+            auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
+            static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            kern<<<grid, 512, lds, g_stream>>>(g);
+        }
         if (g.ws) sp_gemm16_reduce<F16T><<<(uint32_t)(((uint64_t)M * L.N + 255) / 256), 256, 0, g_stream>>>(g, splits);
         return;
     }

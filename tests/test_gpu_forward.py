@@ -280,6 +280,7 @@ def _decoded_layer(S, fmt, N, K, seed):
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
     # a few hundred samples: 256 x 256 tiles with K split over the grid
     ("bf16", 768, 1024, 130), ("f16", 512, 2048, 200), ("bf16", 1024, 1024, 255),
+    ("bf16", 4096, 2048, 65), ("f16", 3000, 4096, 100), ("bf16", 4096, 8192, 128), ("i8", 8192, 2048, 129),
     ("i4", 1024, 2048, 300), ("bf16", 768, 1024, 513), ("i2", 2048, 4096, 1000), ("f16", 512, 1024, 257), ("i8", 1280, 1536, 600),
 ])
 def test_thin_and_split_k_shapes(S, fmt, N, K, n):
