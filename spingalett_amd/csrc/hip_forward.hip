@@ -2516,9 +2516,17 @@ void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float
 }
 
 // K splits of the 256 x 256 GEMM when its tiles would leave compute units idle: at least eight K tiles each
+// Rows of a tile of the big GEMM: up to 128 samples a single row of 128 x 256 tiles instead of half-empty 256 x 256
+// ones; for larger batches the smaller tile was measured and is no faster (256 to 2048 samples, 8192-wide layers).
+uint32_t gemm16_tile_rows(uint32_t M)
+{
+    return M <= 128u ? 128u : 256u;
+}
+
 uint32_t gemm16_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 {
-    const uint32_t tiles = ((M + 255u) / 256u) * ((N + 255u) / 256u), ktiles = K / 64u;
+    const uint32_t bm = gemm16_tile_rows(M);
+    const uint32_t tiles = ((M + bm - 1) / bm) * ((N + 255u) / 256u), ktiles = K / 64u;
     *kper = 0;
     if (tiles >= 192u || ktiles < 16u) return 1;
     uint32_t splits = (256u + tiles - 1) / tiles;
@@ -2680,7 +2688,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
     // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
-    const uint32_t big_tiles = ((M + 255u) / 256u) * ((L.N + 255u) / 256u);
+    const uint32_t bm = gemm16_tile_rows(M);
+    const uint32_t big_tiles = ((M + bm - 1) / bm) * ((L.N + 255u) / 256u);
     const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
     if (aligned && L.K % 64u == 0 && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
@@ -2688,7 +2697,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         else g.ws = ctx.ws;
         const dim3 grid(big_tiles, g.ws ? splits : 1u);
         g_last_kernel = "sp_gemm16_big";
-        if (M <= 128u) {
+        if (bm == 128u) {
             // a single row of tiles: 128 rows instead of 256 half-empty ones
             constexpr size_t lds = 2 * (128 + 256) * 64 * sizeof(uint16_t);
             auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 2, 2>;
