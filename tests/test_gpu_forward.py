@@ -296,6 +296,31 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     net.destroy()
 
 
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        fmt = ["i8", "i4", "i2", "bf16", "f16"][int(rng.integers(0, 5))]
+        N = int(rng.choice([1, 3, 8, 10, 31, 64, 65, 100, 257, 640, 1500]))
+        K = int(rng.choice([8, 24, 64, 136, 256, 520, 1024, 2056, 4096]))
+        n = int(rng.choice([5, 6, 8, 9, 16, 31, 33, 64, 65, 100, 128, 129, 200, 256, 257, 400]))
+        out.append((fmt, N, K, n))
+    return out
+
+
+@pytest.mark.parametrize("fmt,N,K,n", _random_shapes(48, seed=2024))
+def test_seeded_random_layer_shapes(S, fmt, N, K, n):
+    """Shapes drawn around every boundary of the planner (8 / 64 / 128 / 256 samples, 8 / 64 outputs, K below and
+    across chunk sizes, rows that are and are not whole 16-byte units), one layer each, against FP64."""
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N * 7 + K + n)
+    X = np.random.default_rng(n + K).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert rel_max_abs(got, want) <= (8e-3 if fmt == "bf16" else 2e-3)
+    net.destroy()
+
+
 def test_batch_permutation_and_row_independence(S, O):
     """Samples are independent: permuting the batch permutes the outputs bit for bit."""
     src = make_oracle_net(O, [256, 384, 64], ["foo52", "softmax"], seed=31)
