@@ -2550,6 +2550,7 @@ struct ThinPlan {
     bool mode_b;
     bool kw;               // thin operand of <= 8 rows: K split among the waves of a workgroup (sp_skinny16_kw)
     int ncp;               // thin rows held in LDS in that case
+    int nw;                // waves per workgroup in that case (4 or 8)
     uint32_t R, NC;        // streamed rows, thin rows
     int rt, ct;
     uint32_t splits, kper, row_blocks, cblocks;
@@ -2601,7 +2602,9 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
         p.cblocks = 1;
         p.row_blocks = (p.R + 31u) / 32u;
         const uint32_t chunks = (K + bkc - 1) / bkc;
-        uint32_t splits = p.row_blocks >= 384u ? 1u : (512u + p.row_blocks - 1) / p.row_blocks;
+        // 6144 to 12287 streamed rows: eight waves per workgroup instead of a K split across two workgroups
+        p.nw = (p.row_blocks >= 192u && p.row_blocks < 384u && chunks >= 16u) ? 8 : 4;
+        uint32_t splits = p.row_blocks >= 192u ? 1u : (512u + p.row_blocks - 1) / p.row_blocks;
         if (splits > 16u) splits = 16u;
         if (splits > chunks / 4u) splits = chunks / 4u;
         if (splits < 1u) splits = 1u;
@@ -2637,10 +2640,9 @@ void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
     kern<<<dim3(gx, p.splits, 1), 256, lds, g_stream>>>(a);
 }
 
-template <int SFMT, bool F16T, int NCP>
+template <int SFMT, bool F16T, int NCP, int NW>
 void launch_thin_kw(const SkinnyArgs &a, const ThinPlan &p)
 {
-    constexpr int NW = 4;
     constexpr size_t lds = (size_t)NW * 2 * NCP * SkinnyFmt<SFMT>::PITCH + (size_t)NW * (NCP / 2) * 64 * sizeof(float);
     auto kern = sp_skinny16_kw<SFMT, F16T, NCP, NW>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
@@ -2653,7 +2655,7 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
 {
     if (p.splits == 1) a.ws = nullptr;
     if (p.kw) {
-        launch_thin_kw<SFMT, F16T, 8>(a, p);
+        if (p.nw == 8) launch_thin_kw<SFMT, F16T, 8, 8>(a, p); else launch_thin_kw<SFMT, F16T, 8, 4>(a, p);
     } else if (p.rt == 2) {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 2, 2>(a, p); else launch_thin_inst<SFMT, F16T, 2, 1>(a, p);
     } else {
