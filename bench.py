@@ -8,7 +8,7 @@ whose weights were written by the library's own serializer and loaded back
 (load_spingalett keeps the packed arrays; the device computes on them).
 Inputs and outputs are device-resident during the timed region.  One JSON line
 is printed: the headline workload plus, under "workloads", the other
-BASELINE configurations with their own roofline figures and, under "training",
+benchmark configurations (C1, C2, C3, C5) with their own roofline figures and, under "training",
 the reference's published training benchmark (--workload T1 makes that the
 headline instead).
 """
@@ -337,7 +337,7 @@ def main():
     ap.add_argument("--workload", default="C4", choices=sorted(WORKLOADS) + ["T1"],
                     help="C1..C5: forward configurations; T1: the reference's published training benchmark")
     ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
-    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations and the training benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also make one device-to-device copy of the net's arrays (a plain copy kernel of known "
