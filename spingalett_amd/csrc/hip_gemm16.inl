@@ -1,0 +1,601 @@
+// hip_gemm16.inl — the LDS-tiled 16-bit MFMA GEMM for larger batches (sp_gemm16, sp_gemm16_big,
+// sp_gemm16_reduce).  Part of hip_forward.hip's translation unit (included there, inside its unnamed
+// namespace); not compiled on its own.
+
+// ---------------------------------------------------------------------------
+// 16-bit MFMA GEMM (n > 64): C[M][N] = act(bias + scale * A[M][K] . Wq[N][K]^T)
+// ---------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+struct GemmArgs {
+    LayerArgs L;
+    const uint16_t *A;     // [M][K] 16-bit activations
+    void *C;               // [M][N] 16-bit, or FP32 when out_f32
+    uint32_t M;
+    int out_f32;
+    float *ws;             // [splits][M][N] partial sums when the grid splits K (sp_gemm16_big only), else nullptr
+    uint32_t kper;         // k range of one split, a multiple of 64 (0: all of K)
+};
+
+// (float)q as a 16-bit float; exact for |q| <= 128 in either type
+template <bool F16T>
+__device__ __forceinline__ uint32_t int_to_t16(int q)
+{
+    if constexpr (F16T) {
+        _Float16 h = (_Float16)q;
+        uint16_t r;
+        __builtin_memcpy(&r, &h, 2);
+        return r;
+    } else {
+        return __float_as_uint((float)q) >> 16;
+    }
+}
+
+// packed FP16 subtraction a - c (two lanes at once)
+__device__ __forceinline__ uint32_t h2_sub(uint32_t v, uint32_t c)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 a, b;
+    __builtin_memcpy(&a, &v, 4);
+    __builtin_memcpy(&b, &c, 4);
+    a = a - b;
+    uint32_t r;
+    __builtin_memcpy(&r, &a, 4);
+    return r;
+}
+
+// unpack one 32-bit word of codes into 16-bit floats, written as packed pairs (codes 0 1, 2 3, ...)
+template <int FMT, bool F16T>
+__device__ __forceinline__ void unpack_word16(uint32_t w, uint32_t *o)
+{
+    constexpr int bits = fmt_bits(FMT);
+    constexpr int cnt = 32 / bits;
+    if constexpr (F16T && (FMT == I8 || FMT == I4 || FMT == I2)) {
+        // A field masked in place and XORed onto an FP16 constant whose last mantissa bit weighs as much as
+        // the field's lowest bit (the same XOR flips the sign bit: two's complement -> offset binary) reads
+        // as constant + offset + code; one packed subtraction leaves the codes of two fields, exactly.  The
+        // pairs come out as (code k, code k + cnt/2) and a byte permute puts neighbours together.
+        constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;      // low / high halves of two words
+        if constexpr (FMT == I8) {
+            const uint32_t t0 = h2_sub((w & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);            // codes 0, 2
+            const uint32_t t1 = h2_sub(((w >> 8) & 0x00FF00FFu) ^ 0x64806480u, 0x64806480u);     // codes 1, 3
+            o[0] = __builtin_amdgcn_perm(t1, t0, LO);
+            o[1] = __builtin_amdgcn_perm(t1, t0, HI);
+        } else if constexpr (FMT == I4) {
+            const uint32_t y = w >> 8;
+            const uint32_t t0 = h2_sub((w & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);            // codes 0, 4
+            const uint32_t t1 = h2_sub((w & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);            // codes 1, 5
+            const uint32_t t2 = h2_sub((y & 0x000F000Fu) ^ 0x64086408u, 0x64086408u);            // codes 2, 6
+            const uint32_t t3 = h2_sub((y & 0x00F000F0u) ^ 0x54805480u, 0x54805480u);            // codes 3, 7
+            o[0] = __builtin_amdgcn_perm(t1, t0, LO);
+            o[1] = __builtin_amdgcn_perm(t3, t2, LO);
+            o[2] = __builtin_amdgcn_perm(t1, t0, HI);
+            o[3] = __builtin_amdgcn_perm(t3, t2, HI);
+        } else {
+            const uint32_t y = w >> 10;
+            uint32_t p[8];                                                                        // codes k, k + 8
+            p[0] = h2_sub((w & 0x00030003u) ^ 0x64026402u, 0x64026402u);
+            p[1] = h2_sub((w & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);
+            p[2] = h2_sub((w & 0x00300030u) ^ 0x54205420u, 0x54205420u);
+            p[3] = h2_sub((w & 0x00C000C0u) ^ 0x4C804C80u, 0x4C804C80u);
+            p[4] = h2_sub((w & 0x03000300u) ^ 0x46004600u, 0x46004600u);
+            p[5] = h2_sub((y & 0x00030003u) ^ 0x64026402u, 0x64026402u);
+            p[6] = h2_sub((y & 0x000C000Cu) ^ 0x5C085C08u, 0x5C085C08u);
+            p[7] = h2_sub((y & 0x00300030u) ^ 0x54205420u, 0x54205420u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                o[q]     = __builtin_amdgcn_perm(p[2 * q + 1], p[2 * q], LO);
+                o[4 + q] = __builtin_amdgcn_perm(p[2 * q + 1], p[2 * q], HI);
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < cnt; j += 2) {
+        int q0 = (int)(w << (32 - bits - bits * j)) >> (32 - bits);
+        int q1 = (int)(w << (32 - bits - bits * (j + 1))) >> (32 - bits);
+        o[j / 2] = int_to_t16<F16T>(q0) | (int_to_t16<F16T>(q1) << 16);
+    }
+}
+
+// Tile: BM x BN x 64, 256 threads = 2 x 2 waves, each wave TM x TN tiles of 32x32.
+// LDS rows are padded by 8 elements so that 128-bit fragment reads of 32
+// consecutive rows spread over the banks.
+template <int FMT, bool F16T, int TM, int TN, bool ALIGNED>
+__global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
+{
+    constexpr int BM = 64 * TM, BN = 64 * TN, BK = 64, LDK = BK + 8;
+    constexpr int bits = fmt_bits(FMT);
+    constexpr int EPL = 128 / bits;                 // weight elements per 16-byte load
+    constexpr int W_LOADS = (BN * BK / EPL + 255) / 256;
+    constexpr int A_LOADS = BM * BK / 8 / 256;
+
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * LDK];
+
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // tile index: consecutive workgroups go to different XCDs, so give each XCD a
+    // contiguous band of tiles (shared A rows / W rows stay in one L2)
+    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = ntiles / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    const uint32_t tm = bid / tiles_n, tn = bid % tiles_n;
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    uint4 ra[A_LOADS], rw[W_LOADS];
+    const size_t w_row_bytes = (size_t)K * bits / 8u;
+
+    auto load_tiles = [&](uint32_t k0) {
+        if constexpr (ALIGNED) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+                const uint32_t k = k0 + kc * 8;
+                ra[i] = k < K ? *reinterpret_cast<const uint4 *>(g.A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + 256 * i;
+                constexpr int LPR = BK / EPL;           // loads per tile row
+                const int row = c / LPR, kc = c % LPR;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                const uint32_t k = k0 + kc * EPL;
+                const bool ok = (row < BN) && (k < K);
+                rw[i] = ok ? *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)k * bits / 8u)
+                           : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+
+    auto store_tiles = [&](uint32_t k0) {
+        if constexpr (ALIGNED) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                *reinterpret_cast<uint4 *>(&As[row * LDK + kc * 8]) = ra[i];
+            }
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + 256 * i;
+                constexpr int LPR = BK / EPL;
+                const int row = c / LPR, kc = c % LPR;
+                if (row >= BN) continue;
+                uint16_t *dst = &Ws[row * LDK + kc * EPL];
+                if constexpr (FMT == BF16 || FMT == F16) {
+                    *reinterpret_cast<uint4 *>(dst) = rw[i];
+                } else {
+                    const uint32_t w[4] = {rw[i].x, rw[i].y, rw[i].z, rw[i].w};
+                    constexpr int PW = 16 / bits;       // packed pairs per 32-bit word
+                    uint32_t o[4 * PW];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) unpack_word16<FMT, F16T>(w[q], o + q * PW);
+#pragma unroll
+                    for (int v = 0; v < PW; ++v)
+                        *reinterpret_cast<uint4 *>(dst + v * 8) = make_uint4(o[4 * v], o[4 * v + 1], o[4 * v + 2], o[4 * v + 3]);
+                }
+            }
+        } else {
+            // element-wise, fully bounds-checked
+            for (int e = t; e < BM * BK; e += 256) {
+                const int row = e / BK, kk = e % BK;
+                const uint32_t m = m0 + row, k = k0 + kk;
+                As[row * LDK + kk] = (m < M && k < K) ? g.A[(size_t)m * K + k] : (uint16_t)0;
+            }
+            for (int e = t; e < BN * BK; e += 256) {
+                const int row = e / BK, kk = e % BK;
+                const uint32_t n = n0 + row, k = k0 + kk;
+                uint16_t v = 0;
+                if (n < N && k < K) {
+                    const uint64_t idx = (uint64_t)n * K + k;
+                    if constexpr (FMT == BF16 || FMT == F16) v = reinterpret_cast<const uint16_t *>(g.L.w)[idx];
+                    else if constexpr (FMT == F32) v = f32_to_t16<F16T>(reinterpret_cast<const float *>(g.L.w)[idx]);
+                    else v = (uint16_t)int_to_t16<F16T>(int_code<FMT>(g.L.w, idx));
+                }
+                Ws[row * LDK + kk] = v;
+            }
+        }
+    };
+
+    const uint32_t ktiles = (K + BK - 1) / BK;
+    load_tiles(0);
+    for (uint32_t kt = 0; kt < ktiles; ++kt) {
+        __syncthreads();                              // previous tile fully consumed
+        store_tiles(kt * BK);
+        __syncthreads();
+        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
+
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            const int koff = ks + 8 * (lane >> 5);
+            uint4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[i] = *reinterpret_cast<const uint4 *>(&As[(wm * TM * 32 + i * 32 + (lane & 31)) * LDK + koff]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                fb[j] = *reinterpret_cast<const uint4 *>(&Ws[(wn * TN * 32 + j * 32 + (lane & 31)) * LDK + koff]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (F16T) {
+                        f16x8 a, b;
+                        __builtin_memcpy(&a, &fa[i], 16);
+                        __builtin_memcpy(&b, &fb[j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
+                    } else {
+                        bf16x8 a, b;
+                        __builtin_memcpy(&a, &fa[i], 16);
+                        __builtin_memcpy(&b, &fb[j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
+                    }
+                }
+        }
+    }
+
+    // epilogue: scale, bias, activation, store
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= M) continue;
+                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
+                const size_t o = (size_t)row * N + col;
+                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+            }
+        }
+    }
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
+template <int OFF>
+__device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
+
+// 16 bytes per lane from global memory straight into LDS (wave-contiguous 1 KiB at lds_addr):
+// scalar base + 32-bit lane offset, so issuing it costs no vector-ALU instruction.  The compiler
+// does not track these loads: the caller waits with s_waitcnt vmcnt before the data is read.
+__device__ __forceinline__ void lds_dma16(uint32_t lds_addr, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+
+template <int OFF>
+__device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+
+// reads CNT fragments 4 KiB apart (32 tile rows of 128 bytes) starting at addr + BASE
+template <int BASE, int CNT, int I = 0>
+__device__ __forceinline__ void frag_reads(u32x4 *dst, uint32_t addr)
+{
+    if constexpr (I < CNT) {
+        ds_read128<BASE + I * 4096>(dst[I], addr);
+        frag_reads<BASE, CNT, I + 1>(dst, addr);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Large-tile variant of the 16-bit MFMA GEMM (K a multiple of 64, rows 16-byte
+// aligned).  WM x WN waves, each TM x TN tiles of 32x32; BK = 64.
+//   * LDS rows hold 64 elements = eight 16-byte chunks, unpadded; chunk c of row
+//     r sits at position c ^ ((r >> 1) & 7).  A 128-bit fragment read is served 16
+//     lanes (16 consecutive rows, 256 bytes = all 64 banks) per cycle: rows of equal
+//     parity share a 128-byte half, and r >> 1 gives those eight rows eight
+//     different chunk positions.
+//   * 16-bit operands (activations always, BF16/FP16 weights) go from global
+//     memory straight into LDS (global_load_lds_dwordx4: each wave fills 1 KiB =
+//     8 tile rows per instruction); which global chunk a lane fetches carries the
+//     swizzle.  Integer weights pass through registers to be unpacked.
+//   * two LDS stages: tile kt+1 is in flight while tile kt feeds the MFMAs; one
+//     barrier per K tile.
+template <int FMT, bool F16T, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
+{
+    constexpr int NT = 64 * WM * WN, NWAVES = WM * WN;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, BK = 64;
+    constexpr int bits = fmt_bits(FMT);
+    constexpr bool W_DIRECT = (FMT == BF16 || FMT == F16);
+    constexpr int A_ISSUES = BM * 8 / NT;               // 16-byte chunks per thread and tile
+    constexpr int W_ISSUES = BN * 8 / NT;
+    constexpr int EPL = 128 / bits;                     // weight elements per 16-byte global load
+    constexpr int CPL = EPL / 8;                        // LDS chunks produced per global load
+    constexpr int W_LOADS = W_DIRECT ? 1 : (BN * BK / EPL + NT - 1) / NT;
+
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    uint16_t *As = smem;                                // [2][BM][64]
+    uint16_t *Ws = smem + 2 * BM * BK;                  // [2][BN][64]
+
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // tile order: each XCD (workgroup id mod 8) gets a contiguous run of tiles; inside
+    // the run, 8 row tiles x 4 column tiles are consecutive so that the 32 workgroups
+    // an XCD runs at once share A rows and W rows in its L2
+    const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = ntiles / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    uint32_t tm, tn;
+    {
+        constexpr uint32_t GM = 8;
+        const uint32_t group = bid / (GM * tiles_n);
+        const uint32_t first = group * GM;
+        const uint32_t rows = tiles_m - first < GM ? tiles_m - first : GM;
+        const uint32_t in = bid - group * GM * tiles_n;
+        tm = first + in % rows;
+        tn = in / rows;
+    }
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // LDS-DMA sources: a uniform base (advanced per K tile on the scalar unit) plus a fixed 32-bit
+    // byte offset per lane and issue, and LDS destinations derived from a scalar wave index: the main
+    // loop then issues its loads without any vector-ALU instruction, which would otherwise queue
+    // behind the other wave's MFMAs
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    // Only the first wave of each SIMD (waves 0 .. NWAVES/2-1, which the issue arbiter serves first)
+    // issues the loads, for itself and for wave + NWAVES/2: a wave stalls while the address unit takes
+    // its load, and the other wave of the SIMD keeps the MFMA pipe fed meanwhile.
+    constexpr int HALF = NWAVES / 2;
+    constexpr int A_DUTY = 2 * A_ISSUES, W_DUTY = W_DIRECT ? 2 * W_ISSUES : 1;
+    uint32_t a_voff[A_DUTY], w_voff[W_DUTY];
+#pragma unroll
+    for (int d = 0; d < A_DUTY; ++d) {
+        const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+        const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
+        const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+        a_voff[d] = (uint32_t)(((size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
+    }
+    if constexpr (W_DIRECT) {
+#pragma unroll
+        for (int d = 0; d < W_DUTY; ++d) {
+            const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+            const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
+            const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+            w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
+        }
+    }
+    const char *a_base = reinterpret_cast<const char *>(g.A);
+    const char *w_base = reinterpret_cast<const char *>(g.L.w);
+    const size_t w_row_bytes = (size_t)K * bits / 8u;
+    uint4 rw[W_LOADS];
+    const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)As + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
+    const uint32_t lds_w = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)Ws + (uint32_t)(wave_s & (HALF - 1)) * 1024u;
+    const bool loader = wave_s < HALF;
+    // the idx-th load instruction of a loader wave's tile (A first, then W); idx is a constant once
+    // the caller's loops are unrolled
+    constexpr int DMA_TOTAL = A_DUTY + (W_DIRECT ? W_DUTY : 0);
+    auto issue_one = [&](int buf, uint32_t k0, int idx) {
+        if (!loader) return;
+#pragma unroll
+        for (int d = 0; d < A_DUTY; ++d)
+            if (d == idx)
+                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), a_voff[d],
+                          a_base + (size_t)k0 * 2u);
+        if constexpr (W_DIRECT) {
+#pragma unroll
+            for (int d = 0; d < W_DUTY; ++d)
+                if (A_DUTY + d == idx)
+                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), w_voff[d],
+                              w_base + (size_t)k0 * 2u);
+        }
+    };
+    auto issue_direct = [&](int buf, uint32_t k0) {            // the whole tile at once (prologue)
+#pragma unroll
+        for (int idx = 0; idx < DMA_TOTAL; ++idx) issue_one(buf, k0, idx);
+    };
+    auto load_w_regs = [&](uint32_t k0) {
+        if constexpr (!W_DIRECT) {
+            constexpr int LPR = BK / EPL;
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + NT * i, row = c / LPR, kc = c % LPR;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                if (row < BN)
+                    rw[i] = *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)(k0 + kc * EPL) * bits / 8u);
+            }
+        }
+    };
+    auto store_w_regs = [&](int buf) {
+        if constexpr (!W_DIRECT) {
+            constexpr int LPR = BK / EPL;
+            constexpr int PW = 16 / bits;
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + NT * i, row = c / LPR, kc = c % LPR;
+                if (row >= BN) continue;
+                const uint32_t w[4] = {rw[i].x, rw[i].y, rw[i].z, rw[i].w};
+                uint32_t o[4 * PW];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) unpack_word16<FMT, F16T>(w[q], o + q * PW);
+                uint16_t *rowp = Ws + buf * BN * BK + row * BK;
+#pragma unroll
+                for (int v = 0; v < CPL; ++v) {
+                    const int chunk = kc * CPL + v;
+                    *reinterpret_cast<uint4 *>(rowp + ((chunk ^ ((row >> 1) & 7)) << 3)) =
+                        make_uint4(o[4 * v], o[4 * v + 1], o[4 * v + 2], o[4 * v + 3]);
+                }
+            }
+        }
+    };
+
+    // ---- main loop -----------------------------------------------------------
+    // Fragment reads are issued as explicit ds_read_b128 with manual lgkmcnt waits:
+    // the compiler would otherwise drain every pending LDS-DMA load before the first
+    // LDS read of an iteration and serialise load and compute.  Reads of k-step s+1
+    // are in flight while the MFMAs of k-step s run.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)smem;
+    const int h = lane >> 5, l7 = (lane >> 1) & 7;
+    uint32_t va[4], vw[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const uint32_t xo = (uint32_t)(((2 * ks + h) ^ l7) << 4);
+        va[ks] = lds0 + (uint32_t)((wm * TM * 32 + (lane & 31)) * 128) + xo;
+        vw[ks] = lds0 + (uint32_t)(2 * BM * BK * 2) + (uint32_t)((wn * TN * 32 + (lane & 31)) * 128) + xo;
+    }
+    u32x4 fa[2][TM], fb[2][TN];
+
+    // A loader wave slips one load instruction behind each of the first MFMAs of k-steps 0..2: the
+    // matrix pipe is busy for eight passes after every issue, and the address unit takes the load meanwhile.
+    constexpr int DPS = (DMA_TOTAL + 2) / 3;              // load instructions per k-step
+    auto stage = [&](auto cur_c, bool more, uint32_t knext) {
+        constexpr int CUR = decltype(cur_c)::value;
+        if (more) load_w_regs(knext);
+        frag_reads<CUR * BM * BK * 2, TM>(fa[0], va[0]);
+        frag_reads<CUR * BN * BK * 2, TN>(fb[0], vw[0]);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int cs = ks & 1;
+            if (ks < 3) {
+                frag_reads<CUR * BM * BK * 2, TM>(fa[cs ^ 1], va[ks + 1]);
+                frag_reads<CUR * BN * BK * 2, TN>(fb[cs ^ 1], vw[ks + 1]);
+                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+            } else {
+                asm volatile("s_waitcnt lgkmcnt(0)");
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[cs][i]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[cs][j]));
+            __builtin_amdgcn_sched_barrier(0);          // keep the MFMA group between its wait and the next reads
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (F16T) {
+                        f16x8 a, b;
+                        __builtin_memcpy(&a, &fa[cs][i], 16);
+                        __builtin_memcpy(&b, &fb[cs][j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i][j], 0, 0, 0);
+                    } else {
+                        bf16x8 a, b;
+                        __builtin_memcpy(&a, &fa[cs][i], 16);
+                        __builtin_memcpy(&b, &fb[cs][j], 16);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i][j], 0, 0, 0);
+                    }
+                    if (more && ks < 3 && i * TN + j < DPS) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(CUR ^ 1, knext, ks * DPS + i * TN + j);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (more) store_w_regs(CUR ^ 1);
+        asm volatile("s_waitcnt vmcnt(0)");         // this wave's share of the next stage has landed
+        __syncthreads();                             // ... and everybody's; the current stage is free again
+    };
+
+    // grid y splits K for problems with too few tiles to fill the chip
+    const uint32_t kbeg = g.kper ? blockIdx.y * g.kper : 0u;
+    const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
+    const uint32_t ktiles = (kend - kbeg) / BK;
+    issue_direct(0, kbeg);
+    load_w_regs(kbeg);
+    store_w_regs(0);
+    asm volatile("s_waitcnt vmcnt(0)");
+    __syncthreads();
+    for (uint32_t kt = 0; kt < ktiles; kt += 2) {
+        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, kbeg + (kt + 1) * BK);
+        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, kbeg + (kt + 2) * BK);
+    }
+    if (g.ws) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+            if (col >= N) continue;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < M) g.ws[((size_t)blockIdx.y * M + row) * N + col] = acc[i][j][r];
+                }
+        }
+        return;
+    }
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= M) continue;
+                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
+                const size_t o = (size_t)row * N + col;
+                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+            }
+        }
+    }
+}
+
+// adds the K splits of sp_gemm16_big (in split order) and applies scale, bias and activation
+template <bool F16T>
+__global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32_t splits)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)g.M * g.L.N;
+    if (idx >= total) return;
+    float sum = 0.0f;
+    for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
+    const uint32_t col = (uint32_t)(idx % g.L.N);
+    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+    const float v = apply_act(fmaf(sum, g.L.wscale, bias), g.L.act);
+    if (g.out_f32) reinterpret_cast<float *>(g.C)[idx] = v;
+    else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
+}

@@ -1,0 +1,114 @@
+// hip_gemm32.inl — the FP32 MFMA GEMM for FP32 weights beyond 64 samples (sp_gemm32_f32,
+// sp_gemm32_reduce).  Part of hip_forward.hip's translation unit (included there, inside its unnamed
+// namespace); not compiled on its own.
+
+// ---------------------------------------------------------------------------
+// FP32 MFMA GEMM for FP32 weights (n > 64): 64 x 64 x 16 tile, 4 waves
+// ---------------------------------------------------------------------------
+struct Gemm32Args {
+    LayerArgs L;
+    const float *A;
+    float *C;
+    float *ws;             // [splits][M][N] partial sums when the grid splits K, else nullptr
+    uint32_t M;
+    uint32_t kper;         // k range of one split (multiple of 32)
+};
+
+// 64 x 64 x 32 tile, one 32 x 32 MFMA accumulator per wave.  The next K tile is fetched into
+// registers while the current one is multiplied from LDS; small problems split K over grid y
+// (a layer of this path is often a few dozen tiles only) and a second launch adds the parts.
+// VEC: rows are 16-byte aligned (K % 4 == 0) and are read as float4.
+template <bool VEC>
+__global__ __launch_bounds__(256) void sp_gemm32_f32(const Gemm32Args g)
+{
+    constexpr int BM = 64, BN = 64, BK = 32, LDK = BK + 1;
+    __shared__ float As[BM * LDK];
+    __shared__ float Ws[BN * LDK];
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t tiles_n = (N + BN - 1) / BN;
+    const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    const uint32_t kbeg = blockIdx.y * g.kper;
+    const uint32_t kend = kbeg + g.kper < K ? kbeg + g.kper : K;
+    const float *Wf = reinterpret_cast<const float *>(g.L.w);
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+    // each thread carries two 4-element pieces of A and of W per tile: piece p -> row p / 8, k (p % 8) * 4
+    float4 ra[2], rw[2];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int p = t + 256 * i, row = p >> 3;
+            const uint32_t k = k0 + (uint32_t)(p & 7) * 4u;
+            const uint32_t m = m0 + row, n = n0 + row;
+            if constexpr (VEC) {
+                const bool kin = k < kend;                       // whole pieces: K and the split are multiples of 4
+                const float4 va = *reinterpret_cast<const float4 *>(g.A + (size_t)(m < M ? m : M - 1) * K + (kin ? k : 0u));
+                const float4 vw = *reinterpret_cast<const float4 *>(Wf + (size_t)(n < N ? n : N - 1) * K + (kin ? k : 0u));
+                ra[i] = (kin && m < M) ? va : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                rw[i] = (kin && n < N) ? vw : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            } else {
+                float a4[4], w4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const bool kin = k + e < kend;
+                    a4[e] = (kin && m < M) ? g.A[(size_t)m * K + k + e] : 0.0f;
+                    w4[e] = (kin && n < N) ? Wf[(size_t)n * K + k + e] : 0.0f;
+                }
+                ra[i] = make_float4(a4[0], a4[1], a4[2], a4[3]);
+                rw[i] = make_float4(w4[0], w4[1], w4[2], w4[3]);
+            }
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int p = t + 256 * i, row = p >> 3, kk = (p & 7) * 4;
+            float *da = As + row * LDK + kk, *dw = Ws + row * LDK + kk;
+            da[0] = ra[i].x; da[1] = ra[i].y; da[2] = ra[i].z; da[3] = ra[i].w;
+            dw[0] = rw[i].x; dw[1] = rw[i].y; dw[2] = rw[i].z; dw[3] = rw[i].w;
+        }
+    };
+
+    fetch(kbeg);
+    for (uint32_t k0 = kbeg; k0 < kend; k0 += BK) {
+        stash();
+        __syncthreads();
+        if (k0 + BK < kend) fetch(k0 + BK);
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 2) {
+            const float a = As[(wm * 32 + (lane & 31)) * LDK + ks + (lane >> 5)];
+            const float b = Ws[(wn * 32 + (lane & 31)) * LDK + ks + (lane >> 5)];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    const uint32_t col = n0 + wn * 32 + (lane & 31);
+    if (col >= N) return;
+    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const uint32_t row = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row >= M) continue;
+        if (g.ws) g.ws[((size_t)blockIdx.y * M + row) * N + col] = acc[r];
+        else g.C[(size_t)row * N + col] = apply_act(acc[r] + bias, g.L.act);
+    }
+}
+
+// adds the K splits of sp_gemm32_f32 (in split order) and applies bias and activation
+__global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint32_t splits)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t total = (uint64_t)g.M * g.L.N;
+    if (idx >= total) return;
+    float sum = 0.0f;
+    for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
+    const uint32_t col = (uint32_t)(idx % g.L.N);
+    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+    g.C[idx] = apply_act(sum + bias, g.L.act);
+}

@@ -1,0 +1,571 @@
+// hip_gemv.inl — the kernels for 1..4 samples (FP32 weights: up to 64): vector GEMV and the
+// integer GEMV on the INT8 matrix cores.  Part of hip_forward.hip's translation unit (included there,
+// inside its unnamed namespace); not compiled on its own.
+
+// ---------------------------------------------------------------------------
+// GEMV family (n <= 64): y[b][j] = act(bias[j] + scale * sum_k q[j][k] x[b][k])
+// ---------------------------------------------------------------------------
+struct LayerArgs {
+    const uint8_t *w;      // serialized weight codes, row-major [N][K]
+    const uint8_t *bias;   // serialized bias codes [N]
+    float wscale;          // folded weight scale
+    float bscale;          // folded bias scale
+    int bias_fmt;
+    int act;               // activation applied in the epilogue (A_NONE for softmax layers)
+    uint32_t N, K;         // out, in
+};
+
+// unpack one 16-byte chunk into its 128/bits unscaled float values
+template <int FMT>
+__device__ __forceinline__ void unpack16(const uint4 v, float *o)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (FMT == F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = bits_to_float(w[i]);
+    } else if constexpr (FMT == BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i]     = bits_to_float(w[i] << 16);
+            o[2 * i + 1] = bits_to_float(w[i] & 0xFFFF0000u);
+        }
+    } else if constexpr (FMT == F16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            _Float16 lo, hi;
+            uint16_t a = (uint16_t)(w[i] & 0xFFFFu), b = (uint16_t)(w[i] >> 16);
+            __builtin_memcpy(&lo, &a, 2);
+            __builtin_memcpy(&hi, &b, 2);
+            o[2 * i] = (float)lo;
+            o[2 * i + 1] = (float)hi;
+        }
+    } else if constexpr (FMT == I8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[4 * i + j] = (float)((int)(w[i] << (24 - 8 * j)) >> 24);
+    } else if constexpr (FMT == I4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[8 * i + j] = (float)((int)(w[i] << (28 - 4 * j)) >> 28);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o[16 * i + j] = (float)((int)(w[i] << (30 - 2 * j)) >> 30);
+    }
+}
+
+// Aligned path: every row is a whole number of 16-byte chunks.  One wave owns
+// R rows at a time; lane c takes chunks c, c+64, ... of each row, so a wave reads
+// 1 KiB contiguous per row and instruction.  Partial sums meet in a
+// wavefront-shuffle reduction; lane 0 applies scale, bias and activation.
+template <int FMT, int BT, int R>
+__global__ __launch_bounds__(256) void sp_gemv(const LayerArgs L, const float *__restrict__ x,
+                                               float *__restrict__ y, int nb)
+{
+    constexpr int EPC = 128 / fmt_bits(FMT);
+    const int lane = threadIdx.x & 63;
+    const uint32_t wave = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t row0 = wave * R;
+    if (row0 >= L.N) return;
+    const uint32_t nchunks = L.K / EPC;
+    const size_t row_bytes = (size_t)nchunks * 16u;
+
+    const uint8_t *rp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        uint32_t row = row0 + r < L.N ? row0 + r : L.N - 1;
+        rp[r] = L.w + (size_t)row * row_bytes;
+    }
+
+    float acc[R][BT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[r][b] = 0.0f;
+
+    for (uint32_t c = lane; c < nchunks; c += kWave) {
+        uint4 wv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) wv[r] = *reinterpret_cast<const uint4 *>(rp[r] + (size_t)c * 16u);
+        float wf[R][EPC];
+#pragma unroll
+        for (int r = 0; r < R; ++r) unpack16<FMT>(wv[r], wf[r]);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const int bb = b < nb ? b : nb - 1;
+            const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)c * EPC);
+#pragma unroll
+            for (int e = 0; e < EPC / 4; ++e) {
+                float4 xv = xp[e];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    acc[r][b] = fmaf(wf[r][4 * e + 0], xv.x, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 1], xv.y, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 2], xv.z, acc[r][b]);
+                    acc[r][b] = fmaf(wf[r][4 * e + 3], xv.w, acc[r][b]);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[r][b] = wave_sum(acc[r][b]);
+
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = row0 + r;
+            if (row >= L.N) break;
+            const float bias = elem_value_rt(L.bias_fmt, L.bias, row) * L.bscale;
+#pragma unroll
+            for (int b = 0; b < BT; ++b)
+                if (b < nb) y[(size_t)b * L.N + row] = apply_act(fmaf(acc[r][b], L.wscale, bias), L.act);
+        }
+    }
+}
+
+// Generic path: any K, rows may start inside a byte.  One wave per row, one
+// element per lane and step.
+template <int FMT, int BT>
+__global__ __launch_bounds__(256) void sp_gemv_generic(const LayerArgs L, const float *__restrict__ x,
+                                                       float *__restrict__ y, int nb)
+{
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= L.N) return;
+    float acc[BT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+    const uint64_t base = (uint64_t)row * L.K;
+    for (uint32_t k = lane; k < L.K; k += kWave) {
+        const float w = elem_value<FMT>(L.w, base + k);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const int bb = b < nb ? b : nb - 1;
+            acc[b] = fmaf(w, x[(size_t)bb * L.K + k], acc[b]);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BT; ++b) acc[b] = wave_sum(acc[b]);
+    if (lane == 0) {
+        const float bias = elem_value_rt(L.bias_fmt, L.bias, row) * L.bscale;
+#pragma unroll
+        for (int b = 0; b < BT; ++b)
+            if (b < nb) y[(size_t)b * L.N + row] = apply_act(fmaf(acc[b], L.wscale, bias), L.act);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Integer-weight GEMV on the INT8 matrix cores (n <= 64, INT8 / INT4 / INT2)
+// ---------------------------------------------------------------------------
+// The packed codes are (nearly) MFMA operands already: INT8 bytes as they are,
+// INT4 / INT2 after a mask-and-shift that leaves one code per byte.  The FP32
+// activations are turned into exact integers instead of the weights into floats:
+// per sample and K chunk, X = rint(x * 2^p) with |X| < 2^22, written as three
+// balanced base-256 digits d0 + 256 d1 + 65536 d2, each an INT8.  Then
+//     sum_k q_k x_k = 2^-p * (S0 + 256 S1 + 65536 S2),  S_i = sum_k q_k d_i,k
+// and the S_i are exact INT32 dot products from v_mfma_i32_16x16x64_i8.  One
+// 16-row A tile carries four samples (three digit rows + one zero row each), the
+// B operand is 16 weight rows x 64 codes, so a wave needs no reduction across
+// lanes: lane (n, s) ends up holding S0, S1, S2 of output row n and sample s.
+// The unsigned fields of INT4 / INT2 are biased codes (q + 8, q + 2 after an XOR
+// of the sign bits); the bias is removed exactly with sum_k d_i,k.
+//
+// Work split: a wave owns 16 output rows over the whole K; the waves of a
+// workgroup (1, 2 or 4, chosen so that the grid fills the chip) share the digit
+// planes of the current K chunk in LDS.  No workgroup ever waits for another:
+// device-scope fences cost an L2 write-back on this multi-die part.
+struct GemvI8Args {
+    LayerArgs L;
+    const float *x;        // [nb][K] activations (quantise kernel)
+    uint8_t *aq;           // digit planes, see sp_quant_x
+    float *inv;            // [chunks][nb] 2^-p
+    int *dsum;             // [chunks][nb][4] digit sums (bias removal)
+    float *y;              // [nb][N]
+    int nb;
+    uint32_t kc;           // K chunk = one scale block (multiple of the 64-byte block)
+    uint32_t nchunks;      // ceil(K / kc)
+    uint32_t stage_blocks; // 64-byte blocks whose digit planes are held in LDS at a time
+    uint32_t rw, ks;       // waves of a workgroup: row groups x K shares
+    uint32_t meta_bytes;   // LDS bytes of the per-chunk scale records (multiple of 16)
+};
+
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+
+template <int FMT>
+struct I8Fmt {
+    static constexpr int bits = fmt_bits(FMT);
+    static constexpr int KL = 512 / bits;      // codes per 64-byte row segment (one wave load)
+    static constexpr int NMF = KL / 64;        // MFMAs one lane-load feeds
+    static constexpr int WK = 32 / bits;       // codes per 32-bit word
+    static constexpr int BIAS = FMT == I8 ? 0 : FMT == I4 ? 8 : 2;
+};
+
+// Digits of the WK activations that meet one 32-bit weight word.  X = rint(x * scale);
+// X + 0x808080 written in plain base 256 has the balanced digits of X, each offset by
+// 128: gather the bytes per digit, then flip the top bits.  Byte i of the operand word
+// of MFMA u comes from code i * NMF + u.
+template <int FMT>
+__device__ __forceinline__ void quant_word(const float4 (&v)[I8Fmt<FMT>::WK / 4], float scale,
+                                           uint32_t (&d0)[I8Fmt<FMT>::NMF], uint32_t (&d1)[I8Fmt<FMT>::NMF],
+                                           uint32_t (&d2)[I8Fmt<FMT>::NMF], int &ds0, int &ds1, int &ds2)
+{
+    constexpr int WK = I8Fmt<FMT>::WK, NMF = I8Fmt<FMT>::NMF;
+    uint32_t Xo[WK];
+#pragma unroll
+    for (int c4 = 0; c4 < WK / 4; ++c4) {
+        Xo[4 * c4 + 0] = (uint32_t)((int)rintf(v[c4].x * scale) + 0x808080);
+        Xo[4 * c4 + 1] = (uint32_t)((int)rintf(v[c4].y * scale) + 0x808080);
+        Xo[4 * c4 + 2] = (uint32_t)((int)rintf(v[c4].z * scale) + 0x808080);
+        Xo[4 * c4 + 3] = (uint32_t)((int)rintf(v[c4].w * scale) + 0x808080);
+    }
+#pragma unroll
+    for (int u = 0; u < NMF; ++u) {
+        const uint32_t x0 = Xo[u], x1 = Xo[NMF + u], x2 = Xo[2 * NMF + u], x3 = Xo[3 * NMF + u];
+        const uint32_t lo01 = __builtin_amdgcn_perm(x1, x0, 0x05040100u);   // x0.b0 x0.b1 x1.b0 x1.b1
+        const uint32_t lo23 = __builtin_amdgcn_perm(x3, x2, 0x05040100u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(x1, x0, 0x0c060c02u);   // x0.b2 0 x1.b2 0
+        const uint32_t hi23 = __builtin_amdgcn_perm(x3, x2, 0x0c060c02u);
+        d0[u] = __builtin_amdgcn_perm(lo23, lo01, 0x06040200u) ^ 0x80808080u;
+        d1[u] = __builtin_amdgcn_perm(lo23, lo01, 0x07050301u) ^ 0x80808080u;
+        d2[u] = __builtin_amdgcn_perm(hi23, hi01, 0x06040200u) ^ 0x80808080u;
+        ds0 = __builtin_amdgcn_sdot4((int)d0[u], 0x01010101, ds0, false);
+        ds1 = __builtin_amdgcn_sdot4((int)d1[u], 0x01010101, ds1, false);
+        ds2 = __builtin_amdgcn_sdot4((int)d2[u], 0x01010101, ds2, false);
+    }
+}
+
+// One wave quantises one scale chunk (kc <= 2048 codes starting at code kbase) of up to NS
+// samples (rows xr, xr + K, ...; ns of them are real): every lane fetches its words'
+// activations in one batch of loads (quant_load), the wave agrees on the largest magnitude per
+// sample, and each lane converts what it holds (quant_finish).
+// A 64-byte weight segment (block) is spread over 4 lane groups g of 16 bytes = 4 words w;
+// word w holds WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
+//   INT8: 4w+i (u = 0)      INT4: 8w + 2i + u      INT2: 16w + 4i + u
+// of the lane group.  store(sample, block in chunk, u, g, w, d0, d1, d2) receives the operand
+// words; done(sample, {bits of 2^-p, sum d0, sum d1, sum d2}) the scale record (same in every lane).
+template <int FMT, int NS>
+struct QuantRegs {
+    static constexpr int MAXIT = 2048 / (64 * I8Fmt<FMT>::WK);
+    static constexpr int F4 = I8Fmt<FMT>::WK / 4;
+    float4 v[NS][MAXIT][F4];
+    float m[NS];
+};
+
+template <int FMT, int NS>
+__device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *xr, uint32_t K, uint32_t kbase,
+                                           uint32_t kc, int ns, int lane)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, WK = F::WK, F4 = WK / 4, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr uint32_t WPB = KL / WK;                            // words per block (16)
+    const uint32_t iters = kc / (64u * WK);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        q.m[s] = 0.0f;
+        const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+            const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+            const uint32_t kw = kbase + blk * KL + gg * (KL / 4) + w * WK;     // first code of the word
+            const bool valid = (uint32_t)it < iters && kw < K;                  // rows are whole numbers of words
+            const float4 *src = reinterpret_cast<const float4 *>(xs + (valid ? kw : 0u));
+#pragma unroll
+            for (int c = 0; c < F4; ++c) {
+                float4 t = src[c];
+                if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                q.v[s][it][c] = t;
+                q.m[s] = fmaxf(q.m[s], fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+            }
+        }
+    }
+}
+
+template <int FMT, int NS, class Store, class Done>
+__device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32_t kc, int ns, int lane, Store store, Done done)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr uint32_t WPB = KL / WK;
+    const uint32_t iters = kc / (64u * WK);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        if (s >= ns) break;
+        const float amax = wave_max(q.m[s]);
+        int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
+        if (e < -126) e = -126;
+        int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
+        p = p > 126 ? 126 : p;
+        const bool live = amax > 0.0f && amax < 3.0e38f;         // zero, inf and NaN chunks contribute nothing
+        const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
+        int ds0 = 0, ds1 = 0, ds2 = 0;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            if ((uint32_t)it < iters) {
+                const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+                const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+                uint32_t d0[NMF], d1[NMF], d2[NMF];
+                quant_word<FMT>(q.v[s][it], scale, d0, d1, d2, ds0, ds1, ds2);
+#pragma unroll
+                for (int u = 0; u < NMF; ++u) store((uint32_t)s, blk, (uint32_t)u, gg, w, d0[u], d1[u], d2[u]);
+            }
+        }
+        ds0 = wave_sum_i(ds0);
+        ds1 = wave_sum_i(ds1);
+        ds2 = wave_sum_i(ds2);
+        done((uint32_t)s, make_int4(live ? (int)((uint32_t)(127 - p) << 23) : 0, ds0, ds1, ds2));
+    }
+}
+
+// Quantise kernel (n > 4): one wave per sample and scale chunk, four to a workgroup.
+// Output order = the order the A operand is read: per (block, u, g) the planes are stored as
+//   [sample][digit 0..2][16 bytes]
+// i.e. 3 bytes per element and sample; the GEMV kernel copies them verbatim.
+template <int FMT>
+__global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF;
+    const int lane = threadIdx.x & 63;
+    const uint32_t rec = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (rec >= a.nchunks * (uint32_t)a.nb) return;
+    const uint32_t ch = rec / (uint32_t)a.nb, s0 = rec % (uint32_t)a.nb;
+    const uint32_t nblk = a.kc / KL;                         // blocks per chunk (last chunk zero-padded)
+    QuantRegs<FMT, 1> qr;
+    quant_load<FMT, 1>(qr, a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, 1, lane);
+    quant_finish<FMT, 1>(qr, a.kc, 1, lane,
+        [&](uint32_t, uint32_t blk, uint32_t u, uint32_t g, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+            uint8_t *dst = a.aq + (((((size_t)ch * nblk + blk) * NMF + u) * 4 + g) * (size_t)a.nb + s0) * 48 + w * 4;
+            *reinterpret_cast<uint32_t *>(dst) = d0;
+            *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+            *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+        },
+        [&](uint32_t, int4 md) {
+            if (lane == 0) {
+                a.inv[rec] = __int_as_float(md.x);
+                int *d = a.dsum + (size_t)rec * 4;
+                d[0] = md.y; d[1] = md.z; d[2] = md.w; d[3] = 0;
+            }
+        });
+}
+
+// MT = 16-row A tiles (four samples each).  Rows of D that belong to no sample
+// (fourth row of a slot, slots beyond nb) are never read, so their lanes may load
+// anything: they are pointed at the start of the block.
+// The waves of a workgroup are rw row groups x ks K shares (wave = ks_id * rw +
+// rw_id); share ks_id takes the 64-byte blocks ks_id, ks_id + ks, ... of its rows.
+// Weights are fetched in groups of four blocks, the next group in flight while
+// the current one is multiplied; scale chunks are whole numbers of groups.
+//
+// FQ > 0 (n <= FQ <= 4): the workgroup (at most 8 waves) quantises the activations itself,
+// straight into LDS, instead of copying planes a separate launch prepared: every workgroup
+// repeats the (small) job, and the layer costs one launch instead of two.
+template <int FMT, int MT, int FQ>
+__global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF, G = 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    // [nchunks][nb] {2^-p bits, d0 sum, d1 sum, d2 sum}, then the digit planes of one stage:
+    // [stage blocks][NMF][4 g][nb][3][16 bytes]
+    int4 *meta = reinterpret_cast<int4 *>(lds_all);
+    uint8_t *A_lds = lds_all + a.meta_bytes;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t N = a.L.N, K = a.L.K;
+    const int nb = a.nb;
+    const uint32_t rw = a.rw, ks = a.ks, ks_id = (uint32_t)wave / rw, rw_id = (uint32_t)wave % rw;
+    const uint32_t nrow = (blockIdx.x * rw + rw_id) * 16u + (lane & 15);
+    const uint32_t g = lane >> 4;
+    const size_t row_bytes = (size_t)K * F::bits / 8u;
+    const uint8_t *wrow = a.L.w + (size_t)(nrow < N ? nrow : N - 1) * row_bytes + g * 16u + ks_id * 64u;
+    // largest offset (from wrow) whose 16 bytes stay inside the row; reads past it are clamped there
+    // and meet zero digits
+    const int64_t row_last = (int64_t)row_bytes - 16 - (int64_t)(g * 16u + ks_id * 64u);
+    const uint32_t kcb = a.kc / KL;                           // blocks per scale chunk
+    const uint32_t blk_bytes = (uint32_t)NMF * 4u * (uint32_t)nb * 48u;   // digit planes of one block
+    const uint32_t u_bytes = 4u * (uint32_t)nb * 48u;
+    const uint32_t qstep = ks * 64u;                          // byte distance of this wave's consecutive blocks
+    const uint32_t groups_per_chunk = kcb / (ks * G);         // host guarantees divisibility
+    const uint32_t chunks_per_stage = a.stage_blocks / kcb;
+
+    uint32_t a_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t m = lane & 15u, slot = (uint32_t)mt * 4u + (m >> 2), d = m & 3u;
+        a_off[mt] = (slot < (uint32_t)nb && d < 3u) ? ((g * (uint32_t)nb + slot) * 3u + d) * 16u : 0u;
+    }
+
+    float yacc[MT];
+    i32x4v acc[2][MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        yacc[mt] = 0.0f;
+        acc[0][mt] = acc[1][mt] = (i32x4v){0, 0, 0, 0};
+    }
+
+    auto load_blk = [&](uint32_t q) {                          // q-th block of this wave
+        int64_t off = (int64_t)q * qstep;
+        off = off < row_last ? off : row_last;
+        off = off > 0 ? off : 0;
+        return *reinterpret_cast<const uint4 *>(wrow + off);
+    };
+    auto process = [&](const uint4 wv, const uint8_t *rec) {
+        const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+        i32x4v bop[NMF];
+        if constexpr (FMT == I8) {
+            bop[0] = (i32x4v){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        } else if constexpr (FMT == I4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x8 = w[q] ^ 0x88888888u;          // nibble -> q + 8
+                bop[0][q] = (int)(x8 & 0x0F0F0F0Fu);
+                bop[1][q] = (int)((x8 >> 4) & 0x0F0F0F0Fu);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x2 = w[q] ^ 0xAAAAAAAAu;          // field -> q + 2
+                bop[0][q] = (int)(x2 & 0x03030303u);
+                bop[1][q] = (int)((x2 >> 2) & 0x03030303u);
+                bop[2][q] = (int)((x2 >> 4) & 0x03030303u);
+                bop[3][q] = (int)((x2 >> 6) & 0x03030303u);
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < NMF; ++f)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const i32x4v aop = *reinterpret_cast<const i32x4v *>(rec + f * u_bytes + a_off[mt]);
+                acc[f & 1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, bop[f], acc[f & 1][mt], 0, 0, 0);
+            }
+    };
+    auto fold = [&](uint32_t ch) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int s0 = mt * 4 + (int)g;
+            if (s0 < nb) {
+                const int4 md = meta[(size_t)ch * nb + s0];
+                int S0 = acc[0][mt][0] + acc[1][mt][0], S1 = acc[0][mt][1] + acc[1][mt][1], S2 = acc[0][mt][2] + acc[1][mt][2];
+                if (F::BIAS != 0 && ks_id == 0) {       // one K share removes the code bias of the whole chunk
+                    S0 -= F::BIAS * md.y;
+                    S1 -= F::BIAS * md.z;
+                    S2 -= F::BIAS * md.w;
+                }
+                const float tsum = fmaf((float)S2, 65536.0f, fmaf((float)S1, 256.0f, (float)S0));
+                yacc[mt] = fmaf(tsum, __int_as_float(md.x), yacc[mt]);
+            }
+            acc[0][mt] = acc[1][mt] = (i32x4v){0, 0, 0, 0};
+        }
+    };
+
+    // The self-quantising variant requests the activations of its first scale chunk before the
+    // weights: loads complete in order, and the quantiser should not wait behind the weight stream.
+    constexpr int QN = FQ ? FQ : 1;
+    QuantRegs<FMT, QN> qr;
+    const uint32_t spc = ((uint32_t)nb + QN - 1) / QN;         // sample groups per chunk
+    const uint32_t nch_first = chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks;
+    auto unit_load = [&](uint32_t ch0, uint32_t ui) {
+        const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
+        const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
+        quant_load<FMT, QN>(qr, a.x + (size_t)sbase * K, K, (ch0 + chl) * a.kc, a.kc, ns, lane);
+    };
+    if constexpr (FQ != 0) {
+        if ((uint32_t)wave < nch_first * spc) unit_load(0u, (uint32_t)wave);
+    }
+    // then the first weight group (PD groups in flight; two measured slower than one)
+    constexpr int PD = 1;
+    uint4 nxt[PD][G];
+#pragma unroll
+    for (int d = 0; d < PD; ++d)
+#pragma unroll
+        for (int u = 0; u < G; ++u) nxt[d][u] = load_blk((uint32_t)(d * G + u));
+
+    // scale records of all chunks
+    if constexpr (!FQ) {
+        for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
+            const int *d = a.dsum + (size_t)i * 4;
+            meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
+        }
+    }
+
+    uint32_t q = 0;                                            // this wave's block counter
+    for (uint32_t ch0 = 0; ch0 < a.nchunks; ch0 += chunks_per_stage) {
+        const uint32_t nch = ch0 + chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks - ch0;
+        if (ch0) __syncthreads();                             // previous stage fully consumed
+        if constexpr (!FQ) {
+            const uint4 *src = reinterpret_cast<const uint4 *>(a.aq + (size_t)ch0 * kcb * blk_bytes);
+            const uint32_t pieces = nch * kcb * (blk_bytes / 16u);
+            for (uint32_t i = t; i < pieces; i += nthreads) reinterpret_cast<uint4 *>(A_lds)[i] = src[i];
+        } else {
+            // every wave takes whole scale chunks of this stage, FQ samples at once
+            for (uint32_t ui = (uint32_t)wave; ui < nch * spc; ui += nthreads / 64u) {
+                if (ch0 != 0 || ui != (uint32_t)wave) unit_load(ch0, ui);      // the first one is on its way
+                const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
+                const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
+                quant_finish<FMT, QN>(qr, a.kc, ns, lane,
+                    [&](uint32_t s, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+                        uint8_t *dst = A_lds + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + sbase + s) * 48 + w * 4;
+                        *reinterpret_cast<uint32_t *>(dst) = d0;
+                        *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+                        *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+                    },
+                    [&](uint32_t s, int4 md) {
+                        if (lane == 0) meta[(size_t)(ch0 + chl) * nb + sbase + s] = md;
+                    });
+            }
+        }
+        __syncthreads();
+        const uint8_t *rec = A_lds + (size_t)ks_id * blk_bytes;
+        const size_t rstep = (size_t)ks * blk_bytes;
+        for (uint32_t ch = ch0; ch < ch0 + nch; ++ch) {
+            for (uint32_t gi = 0; gi < groups_per_chunk; ++gi) {
+                uint4 cur[G];
+#pragma unroll
+                for (int u = 0; u < G; ++u) cur[u] = nxt[0][u];
+                q += G;
+#pragma unroll
+                for (int d = 0; d + 1 < PD; ++d)
+#pragma unroll
+                    for (int u = 0; u < G; ++u) nxt[d][u] = nxt[d + 1][u];
+#pragma unroll
+                for (int u = 0; u < G; ++u) nxt[PD - 1][u] = load_blk(q + (PD - 1) * G + u);
+#pragma unroll
+                for (int u = 0; u < G; ++u) process(cur[u], rec + (size_t)u * rstep);
+                rec += G * rstep;
+            }
+            fold(ch);
+        }
+    }
+
+    // add the K shares of a row group (in share order) through LDS
+    if (ks > 1) {
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(A_lds);         // [ks][rw][MT][64]
+        if (ks_id > 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) red[(((size_t)ks_id * rw + rw_id) * MT + mt) * 64 + lane] = yacc[mt];
+        }
+        __syncthreads();
+        if (ks_id > 0) return;
+        for (uint32_t o = 1; o < ks; ++o)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) yacc[mt] += red[(((size_t)o * rw + rw_id) * MT + mt) * 64 + lane];
+    }
+
+    if (nrow < N) {
+        const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, nrow) * a.L.bscale;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int s0 = mt * 4 + (int)g;
+            if (s0 < nb) a.y[(size_t)s0 * N + nrow] = apply_act(fmaf(yacc[mt], a.L.wscale, bias), a.L.act);
+        }
+    }
+}
