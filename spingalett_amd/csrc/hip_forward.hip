@@ -875,10 +875,23 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     }
     g.kper = 0;
     g_last_kernel = "sp_gemm16";
-    constexpr int TM = 2, TN = 2, BM = 64 * TM, BN = 64 * TN;
-    const uint32_t grid = ((M + BM - 1) / BM) * ((L.N + BN - 1) / BN);
-    if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
-    else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
+    // This kernel has one LDS stage, so it lives on the number of resident workgroups: the largest of 128 x 128,
+    // 64 x 128 and 64 x 64 tiles that still gives two workgroups per compute unit (measured: 4096 x 512 x 784 INT8
+    // 21.7 / 16.2 / 12.9 us, 8192 x 8192 x 1000 BF16 0.27 / 0.37 / 0.42 ms); the element-wise loads of unaligned
+    // rows always want the smallest (8192 x 8192 x 1000 INT8: 1.90 / 1.69 / 1.51 ms).
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((L.N + bn - 1) / bn); };
+    const int shape = !aligned ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
+    auto go = [&](auto tm_c, auto tn_c) {
+        constexpr int TM = decltype(tm_c)::value, TN = decltype(tn_c)::value;
+        const uint32_t grid = tiles(64 * TM, 64 * TN);
+        if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
+        else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
+    };
+    using I1 = std::integral_constant<int, 1>;
+    using I2c = std::integral_constant<int, 2>;
+    if (shape == 22) go(I2c{}, I2c{});
+    else if (shape == 12) go(I1{}, I2c{});
+    else go(I1{}, I1{});
 }
 
 void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)

@@ -296,6 +296,25 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     net.destroy()
 
 
+@pytest.mark.parametrize("fmt,N,K,n", [
+    # K not a multiple of 64 keeps a layer on the single-stage tiled GEMM; by tile count it runs 64 x 64,
+    # 64 x 128 or 128 x 128 tiles (ragged edges in both directions), rows that are not whole 16-byte units take
+    # the element-wise loads and always 64 x 64
+    ("bf16", 512, 784, 600), ("i8", 1000, 528, 4096), ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096),
+    ("i4", 520, 1056, 300), ("i2", 2048, 1056, 2048),
+    ("i8", 300, 1000, 700), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 512),
+])
+def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
+    X = np.random.default_rng(n + 1).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert S.lib().sphip_layer_kernel_name(net.h, 1, n, 0).decode() == "sp_gemm16"
+    assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
+    net.destroy()
+
+
 def _random_shapes(count, seed):
     rng = np.random.default_rng(seed)
     out = []
