@@ -700,12 +700,15 @@ struct ThinCtx {
     const uint16_t *w16;   // [N][K] 16-bit weights (raw 16-bit formats, or FP16 codes) when N <= 64, else nullptr
     float *ws;             // split-K workspace
     uint64_t ws_floats;
+    void *soft_out;        // softmax layer: where the normalised outputs go if the layer's kernel can do it itself ...
+    int soft_kind;         // ... as 0 FP32, 1 BF16, 2 FP16
+    bool *soft_done;       // ... and whether it did
 };
 
 struct ThinPlan {
     bool use;
     bool mode_b;
-    bool kw;               // thin operand of <= 8 rows: K split among the waves of a workgroup (sp_skinny16_kw)
+    bool kw;               // thin operand of <= 8 rows (<= 16 outputs): K split among the waves of a workgroup (sp_skinny16_kw)
     int ncp;               // thin rows held in LDS in that case
     int nw;                // waves per workgroup in that case (4 or 8)
     uint32_t R, NC;        // streamed rows, thin rows
@@ -750,18 +753,21 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
     // up to 32 MB of streamed bytes, slower beyond (16384 x 16384 INT4 at 8 samples: 40 us against 34 us).
     const uint64_t streamed_bytes = (uint64_t)p.R * K * (uint64_t)fmt_bits(sfmt) / 8u;
     const bool kw_pays = sfmt == I8 || streamed_bytes <= ((sfmt == I4 || sfmt == I2) ? (64ull << 20) : (32ull << 20));
-    if (p.NC <= 8u && kw_pays) {
+    // A classifier head (at most 16 outputs, activations streamed) takes the same kernel with 16 thin rows; up to 32
+    // chunks of K it runs without a K split across workgroups: one launch, and a softmax can be done in its epilogue.
+    const bool head = p.mode_b && p.NC <= 16u;
+    if ((p.NC <= 8u && kw_pays) || head) {
         // one workgroup per 32 streamed rows, its four waves share K; K is split across workgroups as well only
         // when the rows alone do not fill the chip
         p.kw = true;
-        p.ncp = 8;
+        p.ncp = p.NC <= 8u ? 8 : 16;
         p.rt = p.ct = 1;
         p.cblocks = 1;
         p.row_blocks = (p.R + 31u) / 32u;
         const uint32_t chunks = (K + bkc - 1) / bkc;
         // 6144 to 12287 streamed rows: eight waves per workgroup instead of a K split across two workgroups
-        p.nw = (p.row_blocks >= 192u && p.row_blocks < 384u && chunks >= 16u) ? 8 : 4;
-        uint32_t splits = p.row_blocks >= 192u ? 1u : (512u + p.row_blocks - 1) / p.row_blocks;
+        p.nw = (p.ncp == 8 && p.row_blocks >= 192u && p.row_blocks < 384u && chunks >= 16u) ? 8 : 4;
+        uint32_t splits = (p.row_blocks >= 192u || (head && chunks <= 32u)) ? 1u : (512u + p.row_blocks - 1) / p.row_blocks;
         if (splits > 16u) splits = 16u;
         if (splits > chunks / 4u) splits = chunks / 4u;
         if (splits < 1u) splits = 1u;
@@ -812,7 +818,19 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
 {
     if (p.splits == 1) a.ws = nullptr;
     if (p.kw) {
-        if (p.nw == 8) launch_thin_kw<SFMT, F16T, 8, 8>(a, p); else launch_thin_kw<SFMT, F16T, 8, 4>(a, p);
+        bool wide = false;                      // 16 thin rows: classifier heads only, which stream 16-bit activations
+        if constexpr (SFMT == F16 || SFMT == BF16) {
+            if (p.ncp == 16) {
+                launch_thin_kw<SFMT, F16T, 16, 4>(a, p);
+                wide = true;
+            }
+        }
+        if (wide) {
+        } else if (p.nw == 8) {
+            launch_thin_kw<SFMT, F16T, 8, 8>(a, p);
+        } else {
+            launch_thin_kw<SFMT, F16T, 8, 4>(a, p);
+        }
     } else if (p.rt == 2) {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 2, 2>(a, p); else launch_thin_inst<SFMT, F16T, 2, 1>(a, p);
     } else {
@@ -833,6 +851,11 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.row_blocks = tp.row_blocks; a.cblocks = tp.cblocks; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
         g_last_kernel = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
         if (tp.mode_b) {
+            if (ctx.soft_out && tp.kw && tp.splits == 1) {
+                a.soft_out = ctx.soft_out;
+                a.soft_kind = ctx.soft_kind;
+                *ctx.soft_done = true;
+            }
             a.stream = reinterpret_cast<const uint8_t *>(A);
             a.thin = ctx.w16;
             launch_thin<F16T ? F16 : BF16, F16T>(a, tp);
@@ -1060,6 +1083,7 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
         void *main_out = softmax ? (void *)net->soft_tmp : dst;
         const int out_f32 = (reg != R_GEMM16) || is_last || softmax;
         const bool run = !only_layer || only_layer == l;
+        bool soft_done = false;                 // the layer's own kernel wrote the softmax
         if (run) {
             if (reg == R_GEMV) launch_gemv(net, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
@@ -1071,10 +1095,15 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
                 else if (wa.codes16_valid) ctx.w16 = wa.codes16;
                 ctx.ws = net->split_ws;
                 ctx.ws_floats = net->split_cap;
+                if (softmax && !only_layer) {
+                    ctx.soft_out = dst;
+                    ctx.soft_kind = !is_last ? (f16t ? 2 : 1) : 0;
+                    ctx.soft_done = &soft_done;
+                }
                 launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32, ctx);
             }
         }
-        if (softmax && !only_layer) {
+        if (softmax && !only_layer && !soft_done) {
             const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
             sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(net->soft_tmp, dst, kind, n, net->topo[l]);
         }

@@ -27,6 +27,8 @@ struct SkinnyArgs {
     uint32_t kper;           // codes per K split (whole chunks)
     int out_f32;
     int mode_b;              // 0: streamed rows are outputs, thin rows samples; 1: the reverse
+    void *soft_out;          // sp_skinny16_kw, mode_b, no K split: softmax over a sample's outputs goes here instead of C
+    int soft_kind;           // its element type: 0 FP32, 1 BF16, 2 FP16
 };
 
 template <int FMT>
@@ -547,6 +549,43 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     for (int q = 0; q < NQ; ++q) red[(wave * NQ + q) * 64 + lane] = acc[q];
     __syncthreads();
     if (wave != 0 || r_out >= a.R) return;
+    if (a.soft_out) {
+        // the thin rows are all the outputs of sample r_out, half of them in lane n31 and half in lane n31 + 32:
+        // softmax as Activation.c:5-21 (largest logit subtracted, exponentials, one division by their sum)
+        float v[NQ];
+        float m = -3.402823466e+38f;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const uint32_t c = 8u * (q >> 2) + 4u * h + (q & 3);
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += red[(w * NQ + q) * 64 + lane];
+            const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, c < a.NC ? c : 0u) * a.L.bscale;
+            v[q] = c < a.NC ? fmaf(sum, a.L.wscale, bias) : -3.402823466e+38f;
+            m = fmaxf(m, v[q]);
+        }
+        m = fmaxf(m, __shfl_xor(m, 32));
+        float s = 0.0f;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const uint32_t c = 8u * (q >> 2) + 4u * h + (q & 3);
+            v[q] = c < a.NC ? expf(v[q] - m) : 0.0f;
+            s += v[q];
+        }
+        s += __shfl_xor(s, 32);
+        const float inv = s > 0.0f ? 1.0f / s : 1.0f;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const uint32_t c = 8u * (q >> 2) + 4u * h + (q & 3);
+            if (c >= a.NC) continue;
+            const size_t o = (size_t)r_out * a.L.N + c;
+            const float y = v[q] * inv;
+            if (a.soft_kind == 0) reinterpret_cast<float *>(a.soft_out)[o] = y;
+            else if (a.soft_kind == 1) reinterpret_cast<uint16_t *>(a.soft_out)[o] = f32_to_bf16_rne(y);
+            else reinterpret_cast<uint16_t *>(a.soft_out)[o] = f32_to_f16_sat(y);
+        }
+        return;
+    }
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         const uint32_t c = 8u * (q >> 2) + 4u * h + (q & 3);

@@ -197,6 +197,28 @@ def test_config2_int8(S, O, n):
     S.free_network(net)
 
 
+@pytest.mark.parametrize("fmt,topo,acts,n", [
+    # classifier heads of at most 16 outputs: one streaming launch with the K split inside the workgroup; a softmax
+    # is normalised in that kernel's epilogue when K is short enough to need no split across workgroups
+    ("i8", [320, 10], ["softmax"], 5), ("i8", [1000, 10], ["softmax"], 33), ("i4", [1000, 16], ["softmax"], 300),
+    ("bf16", [1000, 9], ["softmax"], 4096), ("f16", [72, 3], ["softmax"], 100), ("i2", [2048, 13], ["softmax"], 64),
+    ("i8", [4096, 12], ["softmax"], 40),                      # more than 32 chunks: K split, reduce, softmax kernel
+    ("i4", [512, 16], ["tanh"], 200), ("bf16", [256, 11], ["none"], 31),                  # heads without softmax
+    ("i8", [256, 12, 64], ["softmax", "relu"], 128), ("bf16", [256, 8, 32], ["softmax", "none"], 77),  # softmax inside the net
+    ("f16", [1000, 17], ["softmax"], 300),                    # 17 outputs: the wide thin kernel, separate softmax
+])
+def test_classifier_heads(S, O, fmt, topo, acts, n):
+    src = make_oracle_net(O, topo, acts, seed=len(topo) * 100 + topo[-1], bias_std=0.1)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    X = np.random.default_rng(n).standard_normal((n, topo[0])).astype(F32)
+    want = ref.forward_batch_f64(X)
+    got = S.forward_batch(net, X)
+    assert rel_max_abs(got, want) <= TOL_MFMA
+    if acts[-1] == "softmax":
+        assert np.allclose(got.sum(axis=1), 1.0, atol=1e-4)
+    S.free_network(net)
+
+
 def test_config1_fp32_batch256(S, O):
     """FP32 weights, batch 256: FP32 arithmetic end to end, 1e-4."""
     src = make_oracle_net(O, [784, 512, 1000, 10], ["relu", "relu", "softmax"], seed=42, bias_std=0.05)
