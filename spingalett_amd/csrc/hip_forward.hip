@@ -942,7 +942,9 @@ uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
     return (ktiles + per - 1) / per;
 }
 
-void launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, float *ws, uint64_t ws_floats)
+// soft_out: the layer is a softmax layer whose normalised outputs belong there; returns true if they were written
+// (a split-K layer of at most 64 outputs: the reduction does it), false if C holds the logits
+bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, float *ws, uint64_t ws_floats, float *soft_out)
 {
     Gemm32Args g{L, A, C, nullptr, M, 0};
     uint32_t splits = gemm32_splits(M, L.N, L.K, &g.kper);
@@ -953,7 +955,12 @@ void launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, flo
     const bool vec = L.K % 4u == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(L.w) & 15u) == 0;
     if (vec) sp_gemm32_f32<true><<<grid, 256, 0, g_stream>>>(g);
     else sp_gemm32_f32<false><<<grid, 256, 0, g_stream>>>(g);
+    if (splits > 1 && soft_out && L.N <= 64u) {
+        sp_gemm32_reduce_softmax<<<(M + 15u) / 16u, 256, 0, g_stream>>>(g, splits, soft_out);
+        return true;
+    }
     if (splits > 1) sp_gemm32_reduce<<<(uint32_t)(((uint64_t)M * L.N + 255) / 256), 256, 0, g_stream>>>(g, splits);
+    return false;
 }
 
 int reserve(sphip_net *net, uint32_t n, bool keep_layers)
@@ -1087,7 +1094,9 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
         if (run) {
             if (reg == R_GEMV) launch_gemv(net, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
-            else if (reg == R_GEMM32) launch_gemm32(L, (const float *)in, (float *)main_out, n, net->split_ws, net->split_cap);
+            else if (reg == R_GEMM32)
+                soft_done = launch_gemm32(L, (const float *)in, (float *)main_out, n, net->split_ws, net->split_cap,
+                                          softmax && !only_layer ? (float *)dst : nullptr);
             else {
                 const DevArray &wa = net->W[l - 1];
                 ThinCtx ctx{};

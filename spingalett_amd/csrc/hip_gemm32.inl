@@ -112,3 +112,44 @@ __global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint
     const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
     g.C[idx] = apply_act(sum + bias, g.L.act);
 }
+
+// The same for a softmax layer of at most 64 outputs: 16 lanes per sample (lane i takes outputs i, i + 16, ...)
+// add the splits of their logits and normalise them together (Activation.c:5-21: largest logit subtracted,
+// exponentials, one division by their sum), so that the layer needs no separate softmax pass.
+__global__ __launch_bounds__(256) void sp_gemm32_reduce_softmax(const Gemm32Args g, uint32_t splits, float *__restrict__ out)
+{
+    const uint32_t row = blockIdx.x * 16u + (threadIdx.x >> 4), sub = threadIdx.x & 15u;
+    const uint32_t N = g.L.N;
+    const uint64_t total = (uint64_t)g.M * N;
+    float v[4];
+    float m = -3.402823466e+38f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t c = sub + 16u * j;
+        const bool valid = row < g.M && c < N;
+        float sum = 0.0f;
+        if (valid) {
+            for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + (uint64_t)row * N + c];
+            sum += elem_value_rt(g.L.bias_fmt, g.L.bias, c) * g.L.bscale;
+        }
+        v[j] = valid ? sum : -3.402823466e+38f;
+        m = fmaxf(m, v[j]);
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t c = sub + 16u * j;
+        v[j] = (row < g.M && c < N) ? expf(v[j] - m) : 0.0f;
+        s += v[j];
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) s += __shfl_xor(s, off);
+    const float inv = s > 0.0f ? 1.0f / s : 1.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t c = sub + 16u * j;
+        if (row < g.M && c < N) out[(uint64_t)row * N + c] = v[j] * inv;
+    }
+}

@@ -239,6 +239,26 @@ def test_config1_fp32_batch256(S, O):
     S.free_network(net)
 
 
+@pytest.mark.parametrize("topo,n", [([200, 3], 100), ([1000, 64], 300), ([520, 65], 257), ([96, 10, 40], 1000),
+                                    ([64, 10], 4096)])
+def test_fp32_softmax_heads(S, O, topo, n):
+    """FP32 weights beyond 64 samples: a softmax layer of at most 64 outputs whose K is split is normalised by the
+    reduction kernel (one thread per sample), wider ones and unsplit ones by the row kernel; 1e-4 either way."""
+    acts = ["softmax"] + ["tanh"] * (len(topo) - 2)
+    src = make_oracle_net(O, topo, acts, seed=topo[0] + n, bias_std=0.2)
+    net = S.new_spingalett(S.LOSS_CROSS_ENTROPY)
+    S.layer(net, topo[0])
+    for l, width in enumerate(topo[1:]):
+        S.layer(net, width, S.ACT_SOFTMAX if l == 0 else S.ACT_TANH, S.WEIGHT_INITIALIZATION_NONE)
+        S.weights_view(net, l)[:] = src.W(l)
+        S.biases_view(net, l)[:] = src.b(l)
+    X = np.random.default_rng(n).standard_normal((n, topo[0])).astype(F32)
+    want = src.forward_batch(X)
+    got = S.forward_batch(net, X)
+    assert rel_max_abs(got, want) <= TOL_VEC
+    S.free_network(net)
+
+
 @pytest.mark.parametrize("fmt,topo,acts,n", [
     ("i4", [1024, 2048, 2048, 512], ["relu", "tanh", "none"], 8),            # config 3 scaled down
     ("i4", [1024, 2048, 2048, 512], ["relu", "tanh", "none"], 64),
