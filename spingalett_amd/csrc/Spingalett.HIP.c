@@ -32,6 +32,30 @@ void sp_hip_release(sp_net *sn)
     }
 }
 
+/* Copies every array of the net (the file's packed ones, else the FP32 host arrays) into the device net. */
+static bool upload_arrays(sp_net *sn, sphip_net *dev)
+{
+    NeuralNetwork *net = &sn->pub;
+    const bool packed = sn->packed_w && sn->packed_b;
+    for (uint32_t l = 0; l + 1 < net->layers; ++l) {
+        int e;
+        if (packed) {
+            e = sphip_upload_array(dev, l, 0, sn->packed_w[l].codes, sn->packed_w[l].bytes, sn->packed_w[l].max_val)
+             || sphip_upload_array(dev, l, 1, sn->packed_b[l].codes, sn->packed_b[l].bytes, sn->packed_b[l].max_val);
+        } else {
+            const size_t wb = (size_t)net->topology[l] * net->topology[l + 1] * sizeof(float);
+            const size_t bb = (size_t)net->topology[l + 1] * sizeof(float);
+            e = sphip_upload_array(dev, l, 0, net->weights + net->weight_offsets[l], wb, 0.0f)
+             || sphip_upload_array(dev, l, 1, net->biases + net->bias_offsets[l], bb, 0.0f);
+        }
+        if (e) {
+            report(SPINGALETT_ERR_ALLOC, "HIP back-end: upload");
+            return false;
+        }
+    }
+    return true;
+}
+
 /* Creates the device net and uploads every array; idempotent. */
 static bool ensure_device(sp_net *sn)
 {
@@ -62,22 +86,9 @@ static bool ensure_device(sp_net *sn)
         report(SPINGALETT_ERR_ALLOC, "HIP back-end: create");
         return false;
     }
-    for (uint32_t l = 0; l + 1 < net->layers; ++l) {
-        int e;
-        if (packed) {
-            e = sphip_upload_array(dev, l, 0, sn->packed_w[l].codes, sn->packed_w[l].bytes, sn->packed_w[l].max_val)
-             || sphip_upload_array(dev, l, 1, sn->packed_b[l].codes, sn->packed_b[l].bytes, sn->packed_b[l].max_val);
-        } else {
-            const size_t wb = (size_t)net->topology[l] * net->topology[l + 1] * sizeof(float);
-            const size_t bb = (size_t)net->topology[l + 1] * sizeof(float);
-            e = sphip_upload_array(dev, l, 0, net->weights + net->weight_offsets[l], wb, 0.0f)
-             || sphip_upload_array(dev, l, 1, net->biases + net->bias_offsets[l], bb, 0.0f);
-        }
-        if (e) {
-            report(SPINGALETT_ERR_ALLOC, "HIP back-end: upload");
-            sphip_destroy(dev);
-            return false;
-        }
+    if (!upload_arrays(sn, dev)) {
+        sphip_destroy(dev);
+        return false;
     }
     sn->dev = dev;
     sn->dev_precision = prec;
@@ -338,7 +349,13 @@ void train_struct_arguments(TrainArgs args)
     /* training works on the FP32 host arrays: a device copy holding a file's packed arrays is replaced */
     if (sn->dev && sn->dev_precision != PRECISION_FLOAT32) sp_hip_release(sn);
     sp_drop_packed(sn);
-    if (sn->dev) sp_hip_release(sn);             /* the host arrays may have been written since the last upload */
+    /* The host arrays may have been written since the last upload: an existing FP32 device net gets them again
+     * (its buffers, and the training buffers an earlier call left, are kept: allocating and freeing them costs more
+     * than the uploads). */
+    if (sn->dev && !upload_arrays(sn, sn->dev)) {
+        sp_hip_release(sn);
+        return;
+    }
     if (!ensure_device(sn)) return;
     if (sphip_train_begin(sn->dev)) {
         report(SPINGALETT_ERR_ALLOC, "HIP back-end: train");
@@ -459,7 +476,8 @@ void train_struct_arguments(TrainArgs args)
         }
     }
     (void)train_download(sn);
-    sphip_train_end(sn->dev);
+    /* no sphip_train_end: the training buffers stay with the device net for the next call and go with it
+     * (free_network, layer(), spingalett_hip_invalidate) */
     free(order);
     sp_aligned_free(bx);
     sp_aligned_free(bt);

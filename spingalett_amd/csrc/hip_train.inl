@@ -518,7 +518,7 @@ int sphip_train_step(sphip_net *net, const float *x, const float *targets, uint3
         d_x = ts->act[0];
         d_t = ts->targets;
     } else if (!on_dev) {
-        HCHECK(hipMemcpyAsync(ts->act[0], x, (size_t)n * net->topo[0] * sizeof(float), hipMemcpyHostToDevice, g_stream));
+        if (upload_from_host(ts->act[0], x, (size_t)n * net->topo[0] * sizeof(float))) return 1;
         HCHECK(hipMemcpyAsync(ts->targets, targets, (size_t)n * width * sizeof(float), hipMemcpyHostToDevice, g_stream));
         d_x = ts->act[0];
         d_t = ts->targets;

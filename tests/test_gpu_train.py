@@ -209,6 +209,48 @@ def test_full_batch_train_matches_oracle_epochs():
     S.free_network(net)
 
 
+def test_repeated_train_calls_pick_up_host_side_edits_and_keep_their_state():
+    """The device net and its training buffers survive a train() call; the next call uploads the host arrays
+    again (they are the caller's to edit), continues the optimizer state, and may bring a different batch size."""
+    topo, acts, loss = [10, 24, 4], ["relu", "softmax"], 1
+    net, onet = public_net(topo, acts, loss, seed=11)
+    rng = np.random.default_rng(3)
+    X = rng.standard_normal((90, topo[0])).astype(np.float32)
+    T = targets_for(rng, 90, topo[-1], True)
+    st = O.TrainState(onet)
+
+    def oracle_epochs(x, t, k):
+        st.beta1_pow = st.beta2_pow = np.float32(1.0)      # the running powers restart with every call (Training.c:684-685)
+        for _ in range(k):
+            gW, gB, _ = onet.batch_gradients(x, t)
+            onet.apply_gradients(st, gW, gB, O.OPT_ADAM, lr=0.01)
+
+    S.clear_error()
+    S.train(net, X, T, 3, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.01)
+    oracle_epochs(X, T, 3)
+    # second call: same net, moments continue (time step 4, 5)
+    S.train(net, X, T, 2, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.01)
+    oracle_epochs(X, T, 2)
+    assert net.contents.time_step == 5
+    for l in range(2):
+        assert rel_max_abs(S.weights_view(net, l), onet.W(l)) <= TOL
+    # the caller edits the host arrays between calls; a larger batch follows
+    S.weights_view(net, 0)[:] *= 0.5
+    S.biases_view(net, 1)[:] += 0.25
+    onet.W(0)[:] *= 0.5
+    onet.b(1)[:] += 0.25
+    X2 = rng.standard_normal((200, topo[0])).astype(np.float32)
+    T2 = targets_for(rng, 200, topo[-1], True)
+    S.train(net, X2, T2, 2, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.01)
+    oracle_epochs(X2, T2, 2)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    for l in range(2):
+        assert rel_max_abs(S.weights_view(net, l), onet.W(l)) <= TOL
+        assert rel_max_abs(S.biases_view(net, l), onet.b(l)) <= TOL
+    assert rel_max_abs(S.forward_batch(net, X2[:7]), onet.forward_batch(X2[:7])) <= TOL
+    S.free_network(net)
+
+
 def test_small_batch_train_learns_xor_and_counts_steps():
     """The reference's sanity problem (Examples/XOR.c:20-64)."""
     net, _ = public_net([2, 8, 1], ["tanh", "sigmoid"], 0, seed=4)
