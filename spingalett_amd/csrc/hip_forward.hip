@@ -904,10 +904,18 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     // 21.7 / 16.2 / 12.9 us, 8192 x 8192 x 1000 BF16 0.27 / 0.37 / 0.42 ms); the element-wise loads of unaligned
     // rows always want the smallest (8192 x 8192 x 1000 INT8: 1.90 / 1.69 / 1.51 ms).
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((L.N + bn - 1) / bn); };
-    const int shape = !aligned ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
+    // integer codes whose rows are whole 32-bit words (not whole 16-byte units) next to aligned activations
+    const bool words = !aligned && L.K % 8u == 0 && ((uint64_t)L.K * fmt_bits(FMT)) % 32u == 0 && (FMT == I8 || FMT == I4 || FMT == I2);
+    const int shape = !(aligned || words) ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
     auto go = [&](auto tm_c, auto tn_c) {
         constexpr int TM = decltype(tm_c)::value, TN = decltype(tn_c)::value;
         const uint32_t grid = tiles(64 * TM, 64 * TN);
+        if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
+            if (words) {
+                sp_gemm16<FMT, F16T, TM, TN, true, true><<<grid, 256, 0, g_stream>>>(g);
+                return;
+            }
+        }
         if (aligned) sp_gemm16<FMT, F16T, TM, TN, true><<<grid, 256, 0, g_stream>>>(g);
         else sp_gemm16<FMT, F16T, TM, TN, false><<<grid, 256, 0, g_stream>>>(g);
     };

@@ -103,14 +103,19 @@ __device__ __forceinline__ void unpack_word16(uint32_t w, uint32_t *o)
 // Tile: BM x BN x 64, 256 threads = 2 x 2 waves, each wave TM x TN tiles of 32x32.
 // LDS rows are padded by 8 elements so that 128-bit fragment reads of 32
 // consecutive rows spread over the banks.
-template <int FMT, bool F16T, int TM, int TN, bool ALIGNED>
+// W4 (integer codes, ALIGNED activations): the weight rows are whole 32-bit words but not whole 16-byte units
+// (784 INT4 codes = 392 bytes): the codes are fetched a word at a time instead of element by element.
+template <int FMT, bool F16T, int TM, int TN, bool ALIGNED, bool W4 = false>
 __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
 {
+    static_assert(!W4 || (ALIGNED && (FMT == I8 || FMT == I4 || FMT == I2)), "word loads: integer codes, aligned activations");
     constexpr int BM = 64 * TM, BN = 64 * TN, BK = 64, LDK = BK + 8;
     constexpr int bits = fmt_bits(FMT);
     constexpr int EPL = 128 / bits;                 // weight elements per 16-byte load
     constexpr int W_LOADS = (BN * BK / EPL + 255) / 256;
     constexpr int A_LOADS = BM * BK / 8 / 256;
+    constexpr int CW = 32 / bits;                   // codes per 32-bit word
+    constexpr int W4_LOADS = (BN * BK / CW + 255) / 256;
 
     __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
     __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * LDK];
@@ -139,7 +144,8 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    uint4 ra[A_LOADS], rw[W_LOADS];
+    uint4 ra[A_LOADS], rw[W4 ? 1 : W_LOADS];
+    uint32_t rw4[W4 ? W4_LOADS : 1];
     const size_t w_row_bytes = (size_t)K * bits / 8u;
 
     auto load_tiles = [&](uint32_t k0) {
@@ -151,16 +157,29 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
                 const uint32_t k = k0 + kc * 8;
                 ra[i] = k < K ? *reinterpret_cast<const uint4 *>(g.A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
             }
+            if constexpr (W4) {
 #pragma unroll
-            for (int i = 0; i < W_LOADS; ++i) {
-                const int c = t + 256 * i;
-                constexpr int LPR = BK / EPL;           // loads per tile row
-                const int row = c / LPR, kc = c % LPR;
-                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
-                const uint32_t k = k0 + kc * EPL;
-                const bool ok = (row < BN) && (k < K);
-                rw[i] = ok ? *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)k * bits / 8u)
-                           : make_uint4(0, 0, 0, 0);
+                for (int i = 0; i < W4_LOADS; ++i) {
+                    const int c = t + 256 * i;
+                    constexpr int LPR = BK / CW;        // words per tile row
+                    const int row = c / LPR, kc = c % LPR;
+                    const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                    const uint32_t k = k0 + kc * CW;
+                    const bool ok = (row < BN) && (k < K);      // K is a whole number of words: k < K means k + CW <= K
+                    rw4[i] = ok ? *reinterpret_cast<const uint32_t *>(g.L.w + (size_t)n * w_row_bytes + (size_t)k * bits / 8u) : 0u;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < W_LOADS; ++i) {
+                    const int c = t + 256 * i;
+                    constexpr int LPR = BK / EPL;           // loads per tile row
+                    const int row = c / LPR, kc = c % LPR;
+                    const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                    const uint32_t k = k0 + kc * EPL;
+                    const bool ok = (row < BN) && (k < K);
+                    rw[i] = ok ? *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)k * bits / 8u)
+                               : make_uint4(0, 0, 0, 0);
+                }
             }
         }
     };
@@ -172,8 +191,28 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
                 const int c = t + 256 * i, row = c >> 3, kc = c & 7;
                 *reinterpret_cast<uint4 *>(&As[row * LDK + kc * 8]) = ra[i];
             }
+            if constexpr (W4) {
 #pragma unroll
-            for (int i = 0; i < W_LOADS; ++i) {
+                for (int i = 0; i < W4_LOADS; ++i) {
+                    const int c = t + 256 * i;
+                    constexpr int LPR = BK / CW;
+                    const int row = c / LPR, kc = c % LPR;
+                    if (row >= BN) continue;
+                    constexpr int PW = 16 / bits;       // packed pairs per 32-bit word: 2, 4 or 8
+                    uint32_t o[PW];
+                    unpack_word16<FMT, F16T>(rw4[i], o);
+                    uint16_t *dst = &Ws[row * LDK + kc * CW];
+                    if constexpr (PW == 2) {
+                        *reinterpret_cast<uint2 *>(dst) = make_uint2(o[0], o[1]);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < PW / 4; ++v)
+                            *reinterpret_cast<uint4 *>(dst + v * 8) = make_uint4(o[4 * v], o[4 * v + 1], o[4 * v + 2], o[4 * v + 3]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < (W4 ? 0 : W_LOADS); ++i) {
                 const int c = t + 256 * i;
                 constexpr int LPR = BK / EPL;
                 const int row = c / LPR, kc = c % LPR;

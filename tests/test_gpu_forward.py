@@ -345,6 +345,9 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     ("bf16", 512, 784, 600), ("i8", 1000, 528, 4096), ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096),
     ("i4", 520, 1056, 300), ("i2", 2048, 1056, 2048),
     ("i8", 300, 1000, 700), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 512),
+    # integer rows that are whole 32-bit words but not whole 16-byte units (784 INT4 codes = 392 bytes): word loads
+    ("i4", 512, 784, 1024), ("i2", 300, 784, 300), ("i8", 1000, 776, 600), ("i4", 520, 1000, 64), ("i2", 2048, 1008, 2048),
+    ("i4", 70, 24, 9), ("i8", 4096, 72, 4096),
 ])
 def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
