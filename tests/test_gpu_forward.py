@@ -385,6 +385,21 @@ def test_seeded_random_layer_shapes(S, fmt, N, K, n):
     net.destroy()
 
 
+def test_large_host_input_goes_up_in_chunks(S):
+    """Host inputs of 16 MB and more are uploaded through a ring of pinned 8 MB chunks filled by several threads;
+    sizes that are no multiple of a chunk, twice in a row (the ring is reused), against FP64 on every row."""
+    net, W, b = _decoded_layer(S, "bf16", 16, 1030, seed=77)
+    for n in (5000, 4200):                                  # 20.6 MB and 17.3 MB
+        X = np.random.default_rng(n).standard_normal((n, 1030)).astype(F32)
+        pre = X.astype(np.float64) @ W.T + b
+        want = np.where(pre > 0, pre, 0.01 * pre)
+        got = net.forward(X)
+        assert rel_max_abs(got, want) <= 4e-3
+        bad = np.abs(got - want).max(axis=1) > 4e-3 * np.abs(want).max()
+        assert not bad.any(), np.nonzero(bad)[0][:10]
+    net.destroy()
+
+
 def test_batch_permutation_and_row_independence(S, O):
     """Samples are independent: permuting the batch permutes the outputs bit for bit."""
     src = make_oracle_net(O, [256, 384, 64], ["foo52", "softmax"], seed=31)
