@@ -574,6 +574,11 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
 {
     constexpr int KL = I8Fmt<FMT>::KL;
     if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq) return false;
+    // Small layers: this kernel's fixed phases (quantising the activations, the barrier, the K-share reduction) cost
+    // more than they save, and the vector kernel, whose time goes with codes x samples, is faster: 512 x 784 INT8
+    // 2.7 against 5.4 us at one sample and 4.4 against 7.3 us at four, 2048 x 2048 4.5 against 6.4 us at one; equal
+    // from about 4 M code-sample products (INT2, whose decode costs more vector instructions: half that).
+    if ((uint64_t)L.N * L.K * n <= (FMT == I2 ? (2ull << 20) : (4ull << 20))) return false;
     if (reinterpret_cast<uintptr_t>(x) & 15u) return false;   // the quantiser reads float4
     const int need = (int)(n + 3) / 4;
     const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
