@@ -148,7 +148,8 @@ SPHIP_API int  sphip_time_layer(sphip_net *const *nets, int count, uint32_t laye
 /* `iters` training steps on device-resident inputs and targets, timed like sphip_time_forward. */
 SPHIP_API int  sphip_time_train_step(sphip_net *net, const float *d_x, const float *d_targets, uint32_t n,
                                      const sphip_train_args *args, int iters, float *ms);
-/* Name of the main kernel the most recent sphip_time_layer call launched. */
+/* Name of the main kernel that a forward of n samples with these flags runs for the given layer (1..layers-1):
+ * the library's routing evaluated without launching anything. */
 SPHIP_API const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n,
                                               uint32_t flags);
 

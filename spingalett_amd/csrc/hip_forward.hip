@@ -84,7 +84,14 @@ int fail_hip(const char *what, hipError_t e)
     } while (0)
 
 hipStream_t g_stream = nullptr;
-const char *g_last_kernel = "";   // main kernel of the most recent layer launch
+// Routing state of the calling thread.  The launch_* functions below decide which kernel a layer takes and launch it;
+// with `dry` set they only decide (nothing is enqueued), which is how sphip_layer_kernel_name answers without side
+// effects.  `name` receives the main kernel of the layer routed last.
+struct RouteState {
+    bool dry = false;
+    const char *name = "";
+};
+thread_local RouteState tl_route;
 constexpr uint32_t kGemvStageBytes = 64u * 1024u;   // LDS budget of one stage of the integer GEMV
 
 std::mutex g_init_mutex;
@@ -194,11 +201,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
     return (uint16_t)(u >> 16);
 }
 
+// FP32 -> FP16: finite values beyond the FP16 range become +-65504 (an activation that large stays finite in the
+// reference's FP32 arithmetic; an infinity here would turn into NaNs in the next layer), infinities and NaNs stay
+// what they are.
 __device__ __forceinline__ uint16_t f32_to_f16_sat(float x)
 {
     if (x != x) return (uint16_t)0x7E00u;
-    x = fminf(fmaxf(x, -65504.0f), 65504.0f);
-    _Float16 h = (_Float16)x;
+    const float c = fminf(fmaxf(x, -65504.0f), 65504.0f);
+    _Float16 h = (_Float16)(fabsf(x) == __builtin_inff() ? x : c);
     uint16_t r;
     __builtin_memcpy(&r, &h, 2);
     return r;
@@ -222,6 +232,13 @@ __device__ __forceinline__ int wave_sum_i(int v)
 {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t wave_max_u(uint32_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
     return v;
 }
 
@@ -537,11 +554,12 @@ template <int FMT>
 void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
 {
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 4u == 0);
+    tl_route.name = aligned ? "sp_gemv" : "sp_gemv_generic";
+    if (tl_route.dry) return;
     for (uint32_t b0 = 0; b0 < n; b0 += 8) {
         const int nb = (int)(n - b0 < 8 ? n - b0 : 8);
         const float *xb = x + (size_t)b0 * L.K;
         float *yb = y + (size_t)b0 * L.N;
-        g_last_kernel = aligned ? "sp_gemv" : "sp_gemv_generic";
         if (aligned) {
             constexpr int R = 2;
             const uint32_t waves = (L.N + R - 1) / R, grid = (waves + 3) / 4;
@@ -561,6 +579,7 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
 template <int FMT, int MT, int FQ = 0>
 void launch_gemv_i8_mt(const GemvI8Args &a, uint32_t grid_x, uint32_t threads, size_t lds)
 {
+    if (tl_route.dry) return;
     auto kern = sp_gemv_i8mfma<FMT, MT, FQ>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024), true);
     (void)once;
@@ -573,7 +592,8 @@ template <int FMT>
 bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
 {
     constexpr int KL = I8Fmt<FMT>::KL;
-    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || !net->aq) return false;
+    // (reserve() gives every integer net its digit-plane buffers for up to 64 samples before anything is launched)
+    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || (!net->aq && !tl_route.dry)) return false;
     // Small layers: this kernel's fixed phases (quantising the activations, the barrier, the K-share reduction) cost
     // more than they save, and the vector kernel, whose time goes with codes x samples, is faster: 512 x 784 INT8
     // 2.7 against 5.4 us at one sample and 4.4 against 7.3 us at four, 2048 x 2048 4.5 against 6.4 us at one; equal
@@ -641,7 +661,7 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     const size_t red_bytes = (size_t)waves * MT * 64u * sizeof(float);
     if (lds < red_bytes) lds = red_bytes;
     lds += a.meta_bytes;
-    g_last_kernel = "sp_gemv_i8mfma";
+    tl_route.name = "sp_gemv_i8mfma";
     if (fused) {
         // samples one wave quantises at once: as many as still leave every wave a unit of work
         const uint32_t cps = stage / kc_blocks;
@@ -652,7 +672,7 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
         else launch_gemv_i8_mt<FMT, 1, 4>(a, grid, waves * 64, lds);
         return true;
     }
-    if (!main_only) sp_quant_x<FMT><<<(a.nchunks * n + 3u) / 4u, 256, 0, g_stream>>>(a);
+    if (!main_only && !tl_route.dry) sp_quant_x<FMT><<<(a.nchunks * n + 3u) / 4u, 256, 0, g_stream>>>(a);
     switch (MT) {
     case 1:  launch_gemv_i8_mt<FMT, 1>(a, grid, waves * 64, lds); break;
     case 2:  launch_gemv_i8_mt<FMT, 2>(a, grid, waves * 64, lds); break;
@@ -801,6 +821,7 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
 template <int SFMT, bool F16T, int RT, int CT>
 void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
 {
+    if (tl_route.dry) return;
     constexpr size_t lds = 2 * 32 * CT * SkinnyFmt<SFMT>::PITCH;
     auto kern = sp_skinny16<SFMT, F16T, RT, CT>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
@@ -812,6 +833,7 @@ void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
 template <int SFMT, bool F16T, int NCP, int NW>
 void launch_thin_kw(const SkinnyArgs &a, const ThinPlan &p)
 {
+    if (tl_route.dry) return;
     constexpr size_t lds = (size_t)NW * 2 * NCP * SkinnyFmt<SFMT>::PITCH + (size_t)NW * (NCP / 2) * 64 * sizeof(float);
     auto kern = sp_skinny16_kw<SFMT, F16T, NCP, NW>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
@@ -842,7 +864,7 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
     } else {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1>(a, p);
     }
-    if (p.splits > 1) {
+    if (p.splits > 1 && !tl_route.dry) {
         const uint64_t total = (uint64_t)a.NC * a.R;
         sp_skinny_reduce<F16T><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(a, p.splits);
     }
@@ -855,7 +877,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
         a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.row_blocks = tp.row_blocks; a.cblocks = tp.cblocks; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
-        g_last_kernel = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
+        tl_route.name = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
         if (tp.mode_b) {
             if (ctx.soft_out && tp.kw && tp.splits == 1) {
                 a.soft_out = ctx.soft_out;
@@ -884,7 +906,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
         else g.ws = ctx.ws;
         const dim3 grid(big_tiles, g.ws ? splits : 1u);
-        g_last_kernel = "sp_gemm16_big";
+        tl_route.name = "sp_gemm16_big";
+        if (tl_route.dry) return;
         if (bm == 128u) {
             // a single row of tiles: 128 rows instead of 256 half-empty ones
             constexpr size_t lds = 2 * (128 + 256) * 64 * sizeof(uint16_t);
@@ -903,7 +926,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         return;
     }
     g.kper = 0;
-    g_last_kernel = "sp_gemm16";
+    tl_route.name = "sp_gemm16";
+    if (tl_route.dry) return;
     // This kernel has one LDS stage, so it lives on the number of resident workgroups: the largest of 128 x 128,
     // 64 x 128 and 64 x 64 tiles that still gives two workgroups per compute unit (measured: 4096 x 512 x 784 INT8
     // 21.7 / 16.2 / 12.9 us, 8192 x 8192 x 1000 BF16 0.27 / 0.37 / 0.42 ms); the element-wise loads of unaligned
@@ -964,7 +988,8 @@ bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, flo
     uint32_t splits = gemm32_splits(M, L.N, L.K, &g.kper);
     if (splits > 1 && (uint64_t)splits * M * L.N > ws_floats) { splits = 1; g.kper = (L.K + 31u) / 32u * 32u; }
     if (splits > 1) g.ws = ws;
-    g_last_kernel = "sp_gemm32_f32";
+    tl_route.name = "sp_gemm32_f32";
+    if (tl_route.dry) return false;
     const dim3 grid(((M + 63) / 64) * ((L.N + 63) / 64), splits);
     const bool vec = L.K % 4u == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(L.w) & 15u) == 0;
     if (vec) sp_gemm32_f32<true><<<grid, 256, 0, g_stream>>>(g);
@@ -1560,9 +1585,30 @@ int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t
 
 const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, uint32_t flags)
 {
-    (void)n; (void)flags;
-    if (!net || layer == 0 || layer >= net->layers) return "";
-    return g_last_kernel;
+    if (!net || layer == 0 || layer >= net->layers || n == 0) return "";
+    // the routing code itself, run without launching: workspaces are taken as reserve() would have sized them and
+    // pointers as aligned, which is how sphip_forward calls it
+    tl_route.dry = true;
+    tl_route.name = "";
+    const LayerArgs L = make_layer_args(net, layer);
+    const float *aligned_ptr = reinterpret_cast<const float *>(uintptr_t{256});     // never dereferenced
+    switch (pick_regime(net, n, flags)) {
+    case R_GEMV:
+        launch_gemv(net, L, aligned_ptr, nullptr, n, false);
+        break;
+    case R_GEMM32:
+        (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
+        break;
+    default: {
+        ThinCtx ctx{};
+        ctx.w16 = reinterpret_cast<const uint16_t *>(aligned_ptr);
+        ctx.ws_floats = ~0ull;
+        launch_gemm16(net->prec, L, reinterpret_cast<const uint16_t *>(aligned_ptr), nullptr, n, 1, ctx);
+        break;
+    }
+    }
+    tl_route.dry = false;
+    return tl_route.name;
 }
 
 }  // extern "C"

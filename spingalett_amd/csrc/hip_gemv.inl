@@ -254,7 +254,7 @@ struct QuantRegs {
     static constexpr int MAXIT = 2048 / (64 * I8Fmt<FMT>::WK);
     static constexpr int F4 = I8Fmt<FMT>::WK / 4;
     float4 v[NS][MAXIT][F4];
-    float m[NS];
+    uint32_t m[NS];      // largest |x| as its bit pattern: orders like the value, and infinities and NaNs sort last
 };
 
 template <int FMT, int NS>
@@ -267,7 +267,7 @@ __device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *x
     const uint32_t iters = kc / (64u * WK);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        q.m[s] = 0.0f;
+        q.m[s] = 0u;
         const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
@@ -281,7 +281,9 @@ __device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *x
                 float4 t = src[c];
                 if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 q.v[s][it][c] = t;
-                q.m[s] = fmaxf(q.m[s], fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+                const uint32_t mx = max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu);
+                const uint32_t mz = max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu);
+                q.m[s] = max(q.m[s], max(mx, mz));
             }
         }
     }
@@ -297,12 +299,16 @@ __device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
         if (s >= ns) break;
-        const float amax = wave_max(q.m[s]);
-        int e = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
+        const uint32_t amax = wave_max_u(q.m[s]);
+        int e = (int)(amax >> 23) - 127;
         if (e < -126) e = -126;
         int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
         p = p > 126 ? 126 : p;
-        const bool live = amax > 0.0f && amax < 3.0e38f;         // zero, inf and NaN chunks contribute nothing
+        // A chunk that holds an infinity or a NaN cannot be written in digits: its record carries a NaN instead of
+        // 2^-p, which turns the sample's sums into NaN, and the epilogue redoes those outputs in FP32 arithmetic so
+        // that infinities and NaNs come out as cblas_sgemv / the FP32 dot product give them (Network.c:229-245).
+        const bool finite = amax < 0x7F800000u;
+        const bool live = amax != 0u && finite;                  // an all-zero chunk contributes nothing
         const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
         int ds0 = 0, ds1 = 0, ds2 = 0;
 #pragma unroll
@@ -319,7 +325,7 @@ __device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32
         ds0 = wave_sum_i(ds0);
         ds1 = wave_sum_i(ds1);
         ds2 = wave_sum_i(ds2);
-        done((uint32_t)s, make_int4(live ? (int)((uint32_t)(127 - p) << 23) : 0, ds0, ds1, ds2));
+        done((uint32_t)s, make_int4(live ? (int)((uint32_t)(127 - p) << 23) : finite ? 0 : 0x7FC00000, ds0, ds1, ds2));
     }
 }
 
@@ -565,7 +571,17 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int s0 = mt * 4 + (int)g;
-            if (s0 < nb) a.y[(size_t)s0 * N + nrow] = apply_act(fmaf(yacc[mt], a.L.wscale, bias), a.L.act);
+            if (s0 >= nb) continue;
+            float dot = yacc[mt];
+            if (dot != dot) {
+                // the sample's input holds an infinity or a NaN (the integer sums themselves are always finite):
+                // plain FP32 multiply-adds over the row, in k order
+                const float *xs = a.x + (size_t)s0 * K;
+                const uint64_t base = (uint64_t)nrow * K;
+                dot = 0.0f;
+                for (uint32_t k = 0; k < K; ++k) dot = fmaf((float)int_code<FMT>(a.L.w, base + k), xs[k], dot);
+            }
+            a.y[(size_t)s0 * N + nrow] = apply_act(fmaf(dot, a.L.wscale, bias), a.L.act);
         }
     }
 }

@@ -355,9 +355,186 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     pre = X.astype(np.float64) @ W.T + b
     want = np.where(pre > 0, pre, 0.01 * pre)
     got = net.forward(X)
-    assert S.lib().sphip_layer_kernel_name(net.h, 1, n, 0).decode() == "sp_gemm16"
+    assert _kernel_of(S, net, n) == "sp_gemm16"
     assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
     net.destroy()
+
+
+def _kernel_of(S, net, n, flags=0):
+    return S.lib().sphip_layer_kernel_name(net.h, 1, n, flags).decode()
+
+
+@pytest.mark.parametrize("fmt,N,K", [
+    ("i2", 8192, 8192),          # the hidden layers of configuration 5
+    ("i4", 16384, 4096),         # the last layer of configuration 3, transposed roles
+    ("i8", 2048, 4096),
+    ("i8", 2061, 2064), ("i4", 4099, 2080), ("i2", 1035, 4160),      # N not a multiple of 16, K not a whole scale chunk
+    ("i8", 60000, 80), ("i4", 30000, 160), ("i2", 9000, 320),        # K just above one 64-byte row segment
+    ("i8", 1500, 6144), ("i4", 3000, 10240), ("i2", 2000, 20480),    # several LDS stages of digit planes
+])
+@pytest.mark.parametrize("n", [1, 2, 3, 4])
+def test_integer_matrix_core_gemv_one_to_four_samples(S, fmt, N, K, n):
+    """Integer weights at one to four samples on layers large enough for the self-quantising INT8 matrix-core
+    GEMV (Network.c:229-245 is what it replaces): the kernel that runs is asserted by name, the outputs are
+    compared with FP64 on the decoded arrays at the vector path's 1e-4."""
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 5 * K)
+    assert _kernel_of(S, net, n) == "sp_gemv_i8mfma"
+    X = (np.random.default_rng(n + K).standard_normal((n, K)) * 1.7).astype(F32)
+    X[0, ::7] *= 1e-3                                   # a wide spread of magnitudes inside one scale chunk
+    X[-1, K // 2:] *= 300.0                             # and chunks of very different scale
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert rel_max_abs(got, want) <= TOL_VEC
+    for i in range(n):                                   # every sample on its own scale
+        assert rel_max_abs(got[i], want[i]) <= TOL_VEC, i
+    net.destroy()
+
+
+@pytest.mark.parametrize("fmt,N,K", [("i8", 4096, 2048), ("i2", 8192, 2048), ("i8", 1030, 1040), ("i2", 2500, 832)])
+@pytest.mark.parametrize("n", [5, 8, 9, 13, 17, 24, 25, 33, 48, 49, 64])
+def test_integer_matrix_core_gemv_forced_up_to_64_samples(S, fmt, N, K, n):
+    """SPHIP_FORCE_GEMV keeps the two-launch form (quantise kernel + planes from memory) reachable up to 64 samples:
+    its 2 .. 16 tile instantiations for INT8 and INT2 (INT4: test_vector_path_batch_sizes), 1e-4 against FP64."""
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + K)
+    # INT2 planes of more than 51 samples exceed the LDS of one fetch group: the vector kernel takes those
+    fits = fmt != "i2" or n <= 51
+    assert _kernel_of(S, net, n, S.SPHIP_FORCE_GEMV) == ("sp_gemv_i8mfma" if fits else "sp_gemv")
+    X = np.random.default_rng(n).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X, S.SPHIP_FORCE_GEMV)
+    assert rel_max_abs(got, want) <= TOL_VEC
+    net.destroy()
+
+
+@pytest.mark.parametrize("fmt,N,K,n,kernel", [
+    # either side of where small layers keep the vector kernel: 4 M code-sample products (INT2: 2 M)
+    ("i8", 2048, 2048, 1, "sp_gemv"), ("i8", 2064, 2048, 1, "sp_gemv_i8mfma"),
+    ("i4", 1024, 1024, 4, "sp_gemv"), ("i4", 1040, 1024, 4, "sp_gemv_i8mfma"),
+    ("i2", 1024, 2048, 1, "sp_gemv"), ("i2", 1040, 2048, 1, "sp_gemv_i8mfma"),
+    ("i2", 1024, 1024, 2, "sp_gemv"), ("i2", 1024, 1024, 3, "sp_gemv_i8mfma"),
+    ("i4", 4096, 2056, 2, "sp_gemv_generic"),          # rows that are not whole 16-byte units
+])
+def test_small_integer_layers_keep_the_vector_kernel(S, fmt, N, K, n, kernel):
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=3 * N + K + n)
+    assert _kernel_of(S, net, n) == kernel
+    X = np.random.default_rng(n + 2).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    assert rel_max_abs(net.forward(X), want) <= TOL_VEC
+    net.destroy()
+
+
+def test_config5_int2_full_size_one_to_four_samples(S, O):
+    """Configuration 5 at its real layer sizes (2048 -> 4 x 8192 -> 1000 softmax, INT2 through the serializer,
+    inputs U[-1,1]) at one to four samples, and one sample through the public forward(), against the oracle."""
+    topo = [2048, 8192, 8192, 8192, 8192, 1000]
+    acts = ["sigmoid", "relu", "relu", "tanh", "softmax"]
+    src = make_oracle_net(O, topo, acts, seed=55)
+    _, ref, net = quantized_pair(O, S, src, "i2")
+    h = S.lib().spingalett_hip_handle(net)
+    X = (np.random.default_rng(56).random((4, 2048), dtype=F32) * 2 - 1)
+    want = ref.forward_batch_f64(X)
+    for n in (1, 2, 3, 4):
+        got = S.forward_batch(net, X[:n])
+        names = [S.lib().sphip_layer_kernel_name(h, l, n, 0).decode() for l in range(1, 6)]
+        assert names[:4] == ["sp_gemv_i8mfma"] * 4, names
+        assert rel_max_abs(got, want[:n]) <= TOL_VEC, n
+        assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+    y = S.forward(net, X[2])
+    assert rel_max_abs(y, want[2]) <= TOL_VEC
+    S.free_network(net)
+
+
+def _same_nonfinite(got, want):
+    """NaNs in the same places, infinities in the same places with the same sign."""
+    return (np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isposinf(got), np.isposinf(want))
+            and np.array_equal(np.isneginf(got), np.isneginf(want)))
+
+
+@pytest.mark.parametrize("fmt,N,K,n,flags,kernel", [
+    ("i8", 2064, 2048, 1, 0, "sp_gemv_i8mfma"), ("i4", 4099, 2080, 3, 0, "sp_gemv_i8mfma"),
+    ("i2", 8192, 8192, 4, 0, "sp_gemv_i8mfma"), ("i8", 1030, 1040, 17, 16, "sp_gemv_i8mfma"),
+    ("i4", 512, 1024, 2, 0, "sp_gemv"), ("bf16", 600, 512, 4, 0, "sp_gemv"), ("i2", 301, 250, 3, 0, "sp_gemv_generic"),
+    ("i4", 16384, 2048, 8, 0, "sp_skinny16_kw"), ("i8", 2100, 2064, 48, 0, "sp_skinny16"),
+    ("f16", 1500, 1000, 77, 0, "sp_skinny16"), ("bf16", 10, 1000, 300, 0, "sp_skinny16_kw"),
+    ("bf16", 1024, 1024, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
+    ("i8", 1000, 528, 700, 0, "sp_gemm16"), ("i4", 257, 100, 513, 0, "sp_gemm16"),
+])
+def test_infinities_and_nans_travel_like_in_fp32(S, fmt, N, K, n, flags, kernel):
+    """The reference's FP32 products propagate non-finite inputs (cblas_sgemv / the FP32 dot product,
+    Network.c:229-245; cblas_sgemm, Training.c:327-333): an infinite input gives +-inf where its weight is
+    positive or negative and NaN where it is zero or where infinities of both signs meet, a NaN input gives
+    NaN everywhere in its sample, and other samples are untouched.  Every kernel family, one layer, against
+    FP64 on the decoded arrays (finite outputs at the path's tolerance)."""
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + K + n)
+    assert _kernel_of(S, net, n, flags) == kernel
+    rng = np.random.default_rng(n + N)
+    X = rng.standard_normal((n, K)).astype(F32)
+    X[0, K // 3] = np.inf                                  # one infinity
+    if n > 1:
+        X[1, 5] = np.nan                                   # one NaN
+    if n > 2:
+        X[2, 1], X[2, K - 1] = np.inf, -np.inf             # both signs in one sample: NaN unless a weight is zero ...
+    if n > 3:
+        X[3, K // 2] = -np.inf
+        X[3, K // 2 + 1] = -np.inf                         # ... two of one sign
+    with np.errstate(invalid="ignore", over="ignore"):
+        pre = np.zeros((n, N))
+        for i in range(n):                                 # row by row: products with zero weights must give NaN
+            pre[i] = (W * X[i].astype(np.float64)).sum(axis=1) + b
+        want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X, flags)
+    assert _same_nonfinite(got, want)
+    fin = np.isfinite(want)
+    assert fin[4:].all() and (n < 2 or not fin[1].any())
+    tol = TOL_VEC if kernel.startswith("sp_gemv") else (4e-3 if fmt == "bf16" else 1e-3)
+    if fin.any():
+        assert np.max(np.abs(got[fin] - want[fin])) <= tol * np.max(np.abs(want[fin]))
+    net.destroy()
+
+
+@pytest.mark.parametrize("fmt,n", [("i8", 1), ("i8", 64), ("i8", 600), ("bf16", 600), ("f32", 100)])
+def test_nonfinite_inputs_through_a_softmax_net(S, O, fmt, n):
+    """Whole nets against the oracle: the sample that carries a NaN or an infinity shows the oracle's pattern after
+    ReLU (NaN -> 0, Activation.c:26) and softmax (Activation.c:5-21: no normalisation when the sum is NaN), the others
+    are unaffected."""
+    src = make_oracle_net(O, [2048, 2064, 10], ["leaky_relu", "softmax"], seed=91)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    X = np.random.default_rng(92).standard_normal((n, 2048)).astype(F32)
+    X[0, 7] = np.inf
+    if n > 1:
+        X[n - 1, 100] = np.nan
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = ref.forward_batch(X)
+    got = S.forward_batch(net, X)
+    assert _same_nonfinite(got, want)
+    fin = np.isfinite(want).all(axis=1)
+    if fin.any():
+        assert rel_max_abs(got[fin], want[fin]) <= tol_for(fmt, n)
+    S.free_network(net)
+
+
+def test_fp16_activation_range_saturates(S, O):
+    """Matrix-core paths of FP16 and integer weights carry FP16 activations between layers: a finite hidden
+    activation beyond +-65504 becomes +-65504 (documented deviation: the reference keeps FP32 activations,
+    Training.c:327-343), so the outputs equal the oracle's on activations clamped to that range; BF16 weights
+    (BF16 activations, FP32's range) and the vector path at up to four samples do not saturate."""
+    src = make_oracle_net(O, [64, 96, 8], ["none", "none"], seed=93, bias_std=0.0)
+    src.W(0)[:] *= 4000.0
+    X = np.random.default_rng(94).standard_normal((40, 64)).astype(F32) * 30
+    for fmt in ("i8", "bf16"):
+        _, ref, net = quantized_pair(O, S, src, fmt)
+        hidden = X.astype(np.float64) @ ref.W(0).astype(np.float64).T + ref.b(0)
+        assert np.abs(hidden).max() > 3 * 65504
+        full = hidden @ ref.W(1).astype(np.float64).T + ref.b(1)
+        clamped = np.clip(hidden, -65504, 65504) @ ref.W(1).astype(np.float64).T + ref.b(1)
+        got = S.forward_batch(net, X)
+        assert np.isfinite(got).all()
+        assert rel_max_abs(got, clamped if fmt == "i8" else full) <= TOL_MFMA
+        assert rel_max_abs(S.forward_batch(net, X[:4]), full[:4]) <= TOL_VEC
+        S.free_network(net)
 
 
 def _random_shapes(count, seed):
