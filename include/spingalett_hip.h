@@ -68,6 +68,19 @@ SPHIP_API int  sphip_upload_array(sphip_net *net, uint32_t l, int which,
  *   weights always compute in FP32 (vector kernels up to n = 64). */
 SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y,
                              uint32_t flags);
+/* sphip_forward for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same kernels and results as sphip_forward with
+ * SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE: d_x [n][in] and d_y [n][out] are device pointers, the call enqueues on the
+ * library's stream and does not wait (sphip_synchronize does).  Everything a forward needs beyond those two and the
+ * net's arrays (activation ping-pong buffers, softmax logits, digit planes of the integer GEMV, partial sums of K
+ * splits, FP16 copies of small integer layers) is laid out in one fixed array of SPHIP_NOALLOC_SCRATCH_BYTES that each
+ * GPU holds from library load until the process ends; the call makes no device or pinned allocation and frees none.
+ * A batch whose workspace exceeds the array is refused with an error that names both sizes (sphip_forward takes it).
+ * Nothing in the array needs clearing between calls: every kernel reads only what this call wrote.  All calls on one
+ * GPU share the array, so two calls that overlap in time (from different threads) race; nets of more than 64 layers
+ * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV only. */
+#define SPHIP_NOALLOC_SCRATCH_BYTES (64u << 20)
+SPHIP_API int  sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags);
 /* The evaluation step that follows batch_forward in the reference's epoch loop, on the device:
  * forward of n samples, then per sample compute_sample_loss (SIMD.c:522-552) and the index of
  * the first largest output, then the batch total (batch_compute_loss, Training.c:421-435;

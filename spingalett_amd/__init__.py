@@ -135,7 +135,7 @@ PUBLIC_SYMBOLS = [
 ]
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
-    "sphip_forward", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
+    "sphip_forward", "sphip_forward_noalloc", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
     "sphip_layer_kernel_name", "sphip_evaluate",
     "sphip_train_begin", "sphip_train_end", "sphip_train_set", "sphip_train_get", "sphip_train_step",
@@ -213,6 +213,8 @@ def lib():
     L.sphip_upload_array.restype = C.c_int
     L.sphip_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32]
     L.sphip_forward.restype = C.c_int
+    L.sphip_forward_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32]
+    L.sphip_forward_noalloc.restype = C.c_int
     L.sphip_forward_layers.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]; L.sphip_forward_layers.restype = C.c_int
     L.sphip_decode.argtypes = [C.c_void_p, C.c_uint32, C.c_int, C.c_int, C.c_void_p]; L.sphip_decode.restype = C.c_int
     L.sphip_synchronize.restype = C.c_int
@@ -498,6 +500,10 @@ class DeviceNet:
     def forward_device(self, d_x: DeviceBuffer, n: int, d_y: DeviceBuffer, flags: int = 0):
         _check(lib().sphip_forward(self.h, d_x.ptr, n, d_y.ptr, flags | SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE),
                "sphip_forward")
+
+    def forward_noalloc(self, d_x: DeviceBuffer, n: int, d_y: DeviceBuffer, flags: int = 0) -> int:
+        """sphip_forward_noalloc; returns its status (the caller reads sphip_last_error_string on failure)."""
+        return lib().sphip_forward_noalloc(self.h, d_x.ptr, n, d_y.ptr, flags)
 
     def decode(self, l: int, which: int, mode: int = DEQUANT_STRICT) -> np.ndarray:
         n = self.topology[l] * self.topology[l + 1] if which == 0 else self.topology[l + 1]

@@ -96,6 +96,29 @@ constexpr uint32_t kGemvStageBytes = 64u * 1024u;   // LDS budget of one stage o
 
 std::mutex g_init_mutex;
 
+// Workspace of sphip_forward_noalloc: one fixed array per GPU, held until the process ends.  Host code never uses the
+// array's name as an address: g_scratch_ptr[device] is what hipGetSymbolAddress returned with that device current.
+constexpr size_t kScratchBytes = SPHIP_NOALLOC_SCRATCH_BYTES;
+constexpr int kScratchDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+unsigned char *g_scratch_ptr[kScratchDevices] = {};
+
+// address of the scratch array on the current device (looked up once per device); caller holds g_init_mutex
+int scratch_lookup(unsigned char **out)
+{
+    int dev = 0;
+    HCHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kScratchDevices) return fail_msg("sphip: device index beyond the scratch table");
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        HCHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail_msg("sphip: hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 // One stream per process (default priority), created at first use; safe to call from several threads.
 int ensure_stream()
 {
@@ -105,6 +128,8 @@ int ensure_stream()
     HCHECK(hipGetDeviceCount(&cnt));
     if (cnt <= 0) return fail_msg("no HIP device");
     HCHECK(hipSetDevice(0));
+    unsigned char *sp = nullptr;
+    if (scratch_lookup(&sp)) return 1;
     HCHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     return 0;
 }
@@ -486,6 +511,19 @@ struct DevArray {
 
 struct sphip_train_state;
 
+// Device memory a forward needs beyond the net's arrays, its input and its output.  A net owns one, grown on demand by
+// reserve(); sphip_forward_noalloc lays one out inside the library's fixed scratch array instead.
+struct Workspace {
+    void *buf[2];                  // ping-pong activation buffers, n x widest layer x 4 bytes each
+    uint8_t *aq;                   // digit planes of the current layer input (two-launch form of the integer GEMV) ...
+    float *aq_inv;                 // ... their scales ...
+    int *aq_dsum;                  // ... and digit sums
+    float *soft_tmp;               // FP32 logits of a softmax layer
+    float *split_ws;               // partial sums of K splits
+    uint64_t split_cap;            // ... and how many floats it holds
+    uint16_t *const *codes16;      // [layers-1]: FP16 copy of the codes of an integer layer with few outputs, or nullptr
+};
+
 struct sphip_net {
     uint32_t layers = 0;
     std::vector<uint32_t> topo;
@@ -517,6 +555,12 @@ struct sphip_net {
     float *eval_buf = nullptr;     // evaluation: outputs, staged targets, per-sample loss / prediction / hit, totals
     uint64_t eval_cap = 0;
     sphip_train_state *train = nullptr;   // gradients, optimizer moments, kept activations (training only)
+    std::vector<uint16_t *> codes16_ptrs; // [layers-1] what Workspace::codes16 points at for the net's own workspace
+
+    Workspace workspace() const
+    {
+        return Workspace{{buf[0], buf[1]}, aq, aq_inv, aq_dsum, soft_tmp, split_ws, split_cap, codes16_ptrs.data()};
+    }
 };
 
 namespace {
@@ -589,11 +633,11 @@ void launch_gemv_i8_mt(const GemvI8Args &a, uint32_t grid_x, uint32_t threads, s
 // Integer formats with 16-byte aligned rows go to the INT8 matrix cores:
 // one quantise launch for the layer's input, then the GEMV proper.
 template <int FMT>
-bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
+bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
 {
     constexpr int KL = I8Fmt<FMT>::KL;
     // (reserve() gives every integer net its digit-plane buffers for up to 64 samples before anything is launched)
-    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || (!net->aq && !tl_route.dry)) return false;
+    if (!rows_aligned(FMT, L.K) || L.K < (uint32_t)KL || (!wk.aq && !tl_route.dry)) return false;
     // Small layers: this kernel's fixed phases (quantising the activations, the barrier, the K-share reduction) cost
     // more than they save, and the vector kernel, whose time goes with codes x samples, is faster: 512 x 784 INT8
     // 2.7 against 5.4 us at one sample and 4.4 against 7.3 us at four, 2048 x 2048 4.5 against 6.4 us at one; equal
@@ -604,7 +648,7 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
     GemvI8Args a{};
     a.L = L; a.x = x; a.y = y; a.nb = (int)n;
-    a.aq = net->aq; a.inv = net->aq_inv; a.dsum = net->aq_dsum;
+    a.aq = wk.aq; a.inv = wk.aq_inv; a.dsum = wk.aq_dsum;
     // waves of a workgroup: rw row groups (sharing the digit planes) x ks K shares
     const uint32_t wave_rows = (L.N + 15) / 16;
     const uint32_t kblocks = (L.K + KL - 1) / KL;
@@ -686,15 +730,15 @@ bool launch_gemv_i8(const sphip_net *net, const LayerArgs &L, const float *x, fl
     return true;
 }
 
-void launch_gemv(const sphip_net *net, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
+void launch_gemv(int prec, const Workspace &wk, const LayerArgs &L, const float *x, float *y, uint32_t n, bool main_only)
 {
-    switch (net->prec) {
+    switch (prec) {
     case F32:  launch_gemv_fmt<F32>(L, x, y, n); break;
     case F16:  launch_gemv_fmt<F16>(L, x, y, n); break;
     case BF16: launch_gemv_fmt<BF16>(L, x, y, n); break;
-    case I8:   if (!launch_gemv_i8<I8>(net, L, x, y, n, main_only)) launch_gemv_fmt<I8>(L, x, y, n); break;
-    case I4:   if (!launch_gemv_i8<I4>(net, L, x, y, n, main_only)) launch_gemv_fmt<I4>(L, x, y, n); break;
-    default:   if (!launch_gemv_i8<I2>(net, L, x, y, n, main_only)) launch_gemv_fmt<I2>(L, x, y, n); break;
+    case I8:   if (!launch_gemv_i8<I8>(wk, L, x, y, n, main_only)) launch_gemv_fmt<I8>(L, x, y, n); break;
+    case I4:   if (!launch_gemv_i8<I4>(wk, L, x, y, n, main_only)) launch_gemv_fmt<I4>(L, x, y, n); break;
+    default:   if (!launch_gemv_i8<I2>(wk, L, x, y, n, main_only)) launch_gemv_fmt<I2>(L, x, y, n); break;
     }
 }
 
@@ -1002,82 +1046,108 @@ bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, flo
     return false;
 }
 
+// What a forward of n samples needs of a Workspace (the same routing decisions as the launch_* functions)
+struct WorkspaceNeed {
+    uint64_t act_floats;       // each of the two ping-pong buffers
+    uint64_t soft_floats;
+    uint64_t plane_bytes;      // digit planes: 4 bytes per element (+ padding of the last chunk) ...
+    uint64_t plane_recs;       // ... and one scale (+ four digit sums) per 64 elements
+    uint64_t split_floats;
+};
+
+// an integer layer with at most 64 outputs streams the activations against an FP16 copy of its codes
+bool layer_wants_codes16(const sphip_net *net, uint32_t l /*1-based*/, uint32_t n)
+{
+    if (net->prec < I8) return false;
+    const ThinPlan tp = plan_thin(net->prec, n, net->topo[l], net->topo[l - 1]);
+    return tp.use && tp.mode_b;
+}
+
+WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n)
+{
+    WorkspaceNeed w{};
+    w.act_floats = (uint64_t)n * net->max_width;
+    for (uint32_t l = 1; l < net->layers; ++l)
+        if (net->act[l - 1] == A_SOFTMAX && (uint64_t)n * net->topo[l] > w.soft_floats) w.soft_floats = (uint64_t)n * net->topo[l];
+    if (n <= 64 && net->prec >= I8) {
+        const uint64_t padded = (uint64_t)n * ((uint64_t)net->max_width + 4096u);
+        w.plane_bytes = padded * 4u;
+        w.plane_recs = padded / 64u + 64u;
+    }
+    for (uint32_t l = 1; l < net->layers; ++l) {
+        const uint32_t N = net->topo[l], K = net->topo[l - 1];
+        uint32_t kper = 0;
+        uint64_t ws = 0;
+        if (net->prec == F32) {
+            if (n <= 64) continue;
+            const uint32_t sp = gemm32_splits(n, N, K, &kper);
+            if (sp > 1) ws = (uint64_t)sp * n * N;
+        } else {
+            const ThinPlan tp = plan_thin(net->prec, n, N, K);
+            if (tp.use) {
+                if (tp.splits > 1) ws = (uint64_t)tp.splits * tp.NC * tp.R;
+            } else {
+                const uint32_t sp = gemm16_splits(n, N, K, &kper);
+                if (sp > 1) ws = (uint64_t)sp * n * N;
+            }
+        }
+        if (ws > w.split_floats) w.split_floats = ws;
+    }
+    return w;
+}
+
+void launch_codes16(int prec, const uint8_t *codes, uint16_t *out, uint64_t count)
+{
+    const uint32_t grid = (uint32_t)((count + 255) / 256);
+    if (prec == I8) sp_codes16<I8><<<grid, 256, 0, g_stream>>>(codes, out, count);
+    else if (prec == I4) sp_codes16<I4><<<grid, 256, 0, g_stream>>>(codes, out, count);
+    else sp_codes16<I2><<<grid, 256, 0, g_stream>>>(codes, out, count);
+}
+
+// grows the net's own workspace to what n samples need
 int reserve(sphip_net *net, uint32_t n, bool keep_layers)
 {
-    const uint64_t need = (uint64_t)n * net->max_width;
-    if (need > net->cap_elems) {
+    const WorkspaceNeed need = workspace_need(net, n);
+    if (need.act_floats > net->cap_elems) {
         for (int i = 0; i < 2; ++i) {
             if (net->buf[i]) { HCHECK(hipFree(net->buf[i])); net->buf[i] = nullptr; }
         }
         net->cap_elems = 0;
-        for (int i = 0; i < 2; ++i) HCHECK(hipMalloc(&net->buf[i], need * sizeof(float)));
-        net->cap_elems = need;
+        for (int i = 0; i < 2; ++i) HCHECK(hipMalloc(&net->buf[i], need.act_floats * sizeof(float)));
+        net->cap_elems = need.act_floats;
     }
-    uint64_t soft = 0;
-    for (uint32_t l = 1; l < net->layers; ++l)
-        if (net->act[l - 1] == A_SOFTMAX && (uint64_t)n * net->topo[l] > soft) soft = (uint64_t)n * net->topo[l];
-    if (soft > net->soft_cap) {
+    if (need.soft_floats > net->soft_cap) {
         if (net->soft_tmp) { HCHECK(hipFree(net->soft_tmp)); net->soft_tmp = nullptr; }
         net->soft_cap = 0;
-        HCHECK(hipMalloc((void **)&net->soft_tmp, soft * sizeof(float)));
-        net->soft_cap = soft;
+        HCHECK(hipMalloc((void **)&net->soft_tmp, need.soft_floats * sizeof(float)));
+        net->soft_cap = need.soft_floats;
     }
-    if (n <= 64 && net->prec >= I8 && n > net->aq_cap_n) {
-        // digit planes of the integer GEMV: 4 bytes per element (+ padding of the last chunk), one scale per chunk
+    if (need.plane_bytes && n > net->aq_cap_n) {
         if (net->aq) { HCHECK(hipFree(net->aq)); HCHECK(hipFree(net->aq_inv)); HCHECK(hipFree(net->aq_dsum)); net->aq = nullptr; }
         net->aq_cap_n = 0;
-        const uint64_t padded = (uint64_t)n * ((uint64_t)net->max_width + 4096u);
-        HCHECK(hipMalloc((void **)&net->aq, padded * 4u));
-        HCHECK(hipMalloc((void **)&net->aq_inv, (padded / 64u + 64u) * sizeof(float)));
-        HCHECK(hipMalloc((void **)&net->aq_dsum, (padded / 64u + 64u) * 4u * sizeof(int)));
+        HCHECK(hipMalloc((void **)&net->aq, need.plane_bytes));
+        HCHECK(hipMalloc((void **)&net->aq_inv, need.plane_recs * sizeof(float)));
+        HCHECK(hipMalloc((void **)&net->aq_dsum, need.plane_recs * 4u * sizeof(int)));
         net->aq_cap_n = n;
         net->aq_valid_layer = 0;
     }
     if (keep_layers && !net->layers_buf)
         HCHECK(hipMalloc((void **)&net->layers_buf, net->slots_total * sizeof(float)));
-    if (net->prec == F32 && n > 64) {
-        uint64_t ws = 0;
-        for (uint32_t l = 1; l < net->layers; ++l) {
-            uint32_t kper = 0;
-            const uint32_t sp = gemm32_splits(n, net->topo[l], net->topo[l - 1], &kper);
-            if (sp > 1 && (uint64_t)sp * n * net->topo[l] > ws) ws = (uint64_t)sp * n * net->topo[l];
-        }
-        if (ws > net->split_cap) {
-            if (net->split_ws) { HCHECK(hipFree(net->split_ws)); net->split_ws = nullptr; }
-            net->split_cap = 0;
-            HCHECK(hipMalloc((void **)&net->split_ws, ws * sizeof(float)));
-            net->split_cap = ws;
-        }
+    if (need.split_floats > net->split_cap) {
+        if (net->split_ws) { HCHECK(hipFree(net->split_ws)); net->split_ws = nullptr; }
+        net->split_cap = 0;
+        HCHECK(hipMalloc((void **)&net->split_ws, need.split_floats * sizeof(float)));
+        net->split_cap = need.split_floats;
     }
-    if (net->prec != F32) {
-        // thin-operand kernel: split-K workspace, and FP16 copies of the codes of layers with few outputs
-        uint64_t ws = 0;
-        for (uint32_t l = 1; l < net->layers; ++l) {
-            const ThinPlan tp = plan_thin(net->prec, n, net->topo[l], net->topo[l - 1]);
-            if (!tp.use) {
-                uint32_t kper = 0;
-                const uint32_t sp = gemm16_splits(n, net->topo[l], net->topo[l - 1], &kper);
-                if (sp > 1 && (uint64_t)sp * n * net->topo[l] > ws) ws = (uint64_t)sp * n * net->topo[l];
-                continue;
-            }
-            if (tp.splits > 1 && (uint64_t)tp.splits * tp.NC * tp.R > ws) ws = (uint64_t)tp.splits * tp.NC * tp.R;
-            DevArray &wa = net->W[l - 1];
-            if (tp.mode_b && net->prec >= I8 && !wa.codes16_valid && wa.uploaded) {
-                if (!wa.codes16) HCHECK(hipMalloc((void **)&wa.codes16, wa.count * sizeof(uint16_t)));
-                const uint32_t grid = (uint32_t)((wa.count + 255) / 256);
-                if (net->prec == I8) sp_codes16<I8><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
-                else if (net->prec == I4) sp_codes16<I4><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
-                else sp_codes16<I2><<<grid, 256, 0, g_stream>>>(wa.base, wa.codes16, wa.count);
-                HCHECK(hipGetLastError());
-                wa.codes16_valid = true;
-            }
+    for (uint32_t l = 1; l < net->layers; ++l) {
+        DevArray &wa = net->W[l - 1];
+        if (layer_wants_codes16(net, l, n) && !wa.codes16_valid && wa.uploaded) {
+            if (!wa.codes16) HCHECK(hipMalloc((void **)&wa.codes16, wa.count * sizeof(uint16_t)));
+            launch_codes16(net->prec, wa.base, wa.codes16, wa.count);
+            HCHECK(hipGetLastError());
+            wa.codes16_valid = true;
         }
-        if (ws > net->split_cap) {
-            if (net->split_ws) { HCHECK(hipFree(net->split_ws)); net->split_ws = nullptr; }
-            net->split_cap = 0;
-            HCHECK(hipMalloc((void **)&net->split_ws, ws * sizeof(float)));
-            net->split_cap = ws;
-        }
+        net->codes16_ptrs[l - 1] = wa.codes16_valid ? wa.codes16 : nullptr;
     }
     return 0;
 }
@@ -1102,8 +1172,8 @@ int check_uploaded(const sphip_net *net)
 // Enqueues every kernel of one forward.  d_x, d_y are device pointers.
 // only_layer != 0 restricts the launch to the main kernel of that layer.
 // keep (n == 1): every layer's output goes to its slot of layers_buf, d_x must be slot 0 and d_y the last slot.
-int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags, uint32_t only_layer,
-                    bool keep = false)
+int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint32_t n, float *d_y, uint32_t flags,
+                    uint32_t only_layer, bool keep = false)
 {
     const Regime reg = pick_regime(net, n, flags);
     const bool f16t = net->prec != BF16;          // 16-bit activation type of the matrix-core path
@@ -1113,36 +1183,36 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
     if (reg == R_GEMM16 && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         const uint32_t grid = (uint32_t)((cnt / 4 + 255) / 256 + 1);
-        if (f16t) sp_cvt16<true><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)net->buf[1], cnt);
-        else sp_cvt16<false><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)net->buf[1], cnt);
-        in = net->buf[1];
+        if (f16t) sp_cvt16<true><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
+        else sp_cvt16<false><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
+        in = wk.buf[1];
     } else if (reg == R_GEMM16) {
-        in = net->buf[1];
+        in = wk.buf[1];
     }
 
     for (uint32_t l = 1; l <= last; ++l) {
         const LayerArgs L = make_layer_args(net, l);
         const bool softmax = net->act[l - 1] == A_SOFTMAX;
         const bool is_last = l == last;
-        void *dst = is_last ? (void *)d_y : keep ? (void *)(net->layers_buf + net->slot_off[l]) : net->buf[(l + 1) & 1];
+        void *dst = is_last ? (void *)d_y : keep ? (void *)(net->layers_buf + net->slot_off[l]) : wk.buf[(l + 1) & 1];
         // logits of a softmax layer go to FP32 scratch first
-        void *main_out = softmax ? (void *)net->soft_tmp : dst;
+        void *main_out = softmax ? (void *)wk.soft_tmp : dst;
         const int out_f32 = (reg != R_GEMM16) || is_last || softmax;
         const bool run = !only_layer || only_layer == l;
         bool soft_done = false;                 // the layer's own kernel wrote the softmax
         if (run) {
-            if (reg == R_GEMV) launch_gemv(net, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
+            if (reg == R_GEMV) launch_gemv(net->prec, wk, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
             else if (reg == R_GEMM32)
-                soft_done = launch_gemm32(L, (const float *)in, (float *)main_out, n, net->split_ws, net->split_cap,
+                soft_done = launch_gemm32(L, (const float *)in, (float *)main_out, n, wk.split_ws, wk.split_cap,
                                           softmax && !only_layer ? (float *)dst : nullptr);
             else {
                 const DevArray &wa = net->W[l - 1];
                 ThinCtx ctx{};
                 if (net->prec == F16 || net->prec == BF16) ctx.w16 = reinterpret_cast<const uint16_t *>(wa.base);
-                else if (wa.codes16_valid) ctx.w16 = wa.codes16;
-                ctx.ws = net->split_ws;
-                ctx.ws_floats = net->split_cap;
+                else ctx.w16 = wk.codes16[l - 1];
+                ctx.ws = wk.split_ws;
+                ctx.ws_floats = wk.split_cap;
                 if (softmax && !only_layer) {
                     ctx.soft_out = dst;
                     ctx.soft_kind = !is_last ? (f16t ? 2 : 1) : 0;
@@ -1153,7 +1223,7 @@ int enqueue_forward(sphip_net *net, const float *d_x, uint32_t n, float *d_y, ui
         }
         if (softmax && !only_layer && !soft_done) {
             const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
-            sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(net->soft_tmp, dst, kind, n, net->topo[l]);
+            sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(wk.soft_tmp, dst, kind, n, net->topo[l]);
         }
         in = dst;
     }
@@ -1191,6 +1261,7 @@ int sphip_create(const sphip_desc *desc, sphip_net **out)
     net->prec = desc->precision;
     net->W.resize(desc->layers - 1);
     net->B.resize(desc->layers - 1);
+    net->codes16_ptrs.assign(desc->layers - 1, nullptr);
     for (uint32_t l = 0; l < desc->layers; ++l) {
         if (net->topo[l] > net->max_width) net->max_width = net->topo[l];
         net->total_neurons += net->topo[l];
@@ -1374,13 +1445,68 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
             d_y = net->stage_y;
         }
     }
-    if (enqueue_forward(net, d_x, n, d_y, flags, 0)) return 1;
+    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags, 0)) return 1;
     if (!(flags & SPHIP_Y_ON_DEVICE)) {
         if (!y_pinned) HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
         HCHECK(hipStreamSynchronize(g_stream));
         if (y_pinned) memcpy(y, net->pin_out, out_cnt * sizeof(float));
     }
     return 0;
+}
+
+int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags)
+{
+    if (!net || !d_x || !d_y || n == 0) return fail_msg("sphip_forward_noalloc: invalid argument");
+    if (check_uploaded(net)) return 1;
+    if (!g_stream) return fail_msg("sphip_forward_noalloc: library not initialised");    // sphip_create did it
+    constexpr uint32_t kMaxLayers = 64;
+    if (net->layers > kMaxLayers) return fail_msg("sphip_forward_noalloc: more than 64 layers");
+    unsigned char *base = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_init_mutex);
+        if (scratch_lookup(&base)) return 1;
+    }
+    // lay the workspace out inside the scratch array, every piece at a multiple of 256 bytes
+    const WorkspaceNeed need = workspace_need(net, n);
+    size_t used = 0;
+    auto take = [&](uint64_t bytes) -> unsigned char * {
+        unsigned char *p = base + used;
+        used += (size_t)((bytes + 255u) & ~(uint64_t)255u);
+        return p;
+    };
+    uint16_t *codes[kMaxLayers] = {};
+    Workspace wk{};
+    wk.buf[0] = take(need.act_floats * sizeof(float));
+    wk.buf[1] = take(need.act_floats * sizeof(float));
+    wk.soft_tmp = reinterpret_cast<float *>(take(need.soft_floats * sizeof(float)));
+    if (need.plane_bytes) {
+        wk.aq = take(need.plane_bytes);
+        wk.aq_inv = reinterpret_cast<float *>(take(need.plane_recs * sizeof(float)));
+        wk.aq_dsum = reinterpret_cast<int *>(take(need.plane_recs * 4u * sizeof(int)));
+    }
+    wk.split_ws = reinterpret_cast<float *>(take(need.split_floats * sizeof(float)));
+    wk.split_cap = need.split_floats;
+    // an integer layer with few outputs reads an FP16 copy of its codes: the net's own if an earlier call made one,
+    // else one made here, in the scratch array, on every call
+    bool fresh[kMaxLayers] = {};
+    for (uint32_t l = 1; l < net->layers; ++l) {
+        if (!layer_wants_codes16(net, l, n)) continue;
+        const DevArray &wa = net->W[l - 1];
+        if (wa.codes16_valid) { codes[l - 1] = wa.codes16; continue; }
+        codes[l - 1] = reinterpret_cast<uint16_t *>(take(wa.count * sizeof(uint16_t)));
+        fresh[l - 1] = true;
+    }
+    wk.codes16 = codes;
+    if (used > kScratchBytes) {
+        snprintf(g_err, sizeof g_err, "sphip_forward_noalloc: %u samples of this net need %zu bytes of workspace, the fixed scratch array holds %zu",
+                 n, used, kScratchBytes);
+        return 1;
+    }
+    for (uint32_t l = 1; l < net->layers; ++l)
+        if (fresh[l - 1]) launch_codes16(net->prec, net->W[l - 1].base, codes[l - 1], net->W[l - 1].count);
+    // the integer GEMV's quantise launch is never skipped here (that shortcut belongs to the layer timer)
+    net->aq_valid_layer = 0;
+    return enqueue_forward(net, wk, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0);
 }
 
 int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
@@ -1393,7 +1519,7 @@ int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
     if (grow_pinned(&net->pin_out, &net->pin_out_cap, net->total_neurons)) return 1;
     memcpy(net->pin_in, x, (size_t)net->topo[0] * sizeof(float));
     sp_copy32<<<(net->topo[0] + 255) / 256, 256, 0, g_stream>>>(net->pin_in, net->layers_buf, net->topo[0]);
-    if (enqueue_forward(net, net->layers_buf, 1, net->layers_buf + net->slot_off[last], 0, 0, true)) return 1;
+    if (enqueue_forward(net, net->workspace(), net->layers_buf, 1, net->layers_buf + net->slot_off[last], 0, 0, true)) return 1;
     // all slots, densely packed, straight into pinned memory
     uint32_t dense = 0;
     for (uint32_t l0 = 0; l0 < net->layers; l0 += 16) {
@@ -1446,7 +1572,7 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
         HCHECK(hipMemcpyAsync(d_t, targets, out_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
         d_x = net->stage_x;
     }
-    if (enqueue_forward(net, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0)) return 1;
+    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0)) return 1;
     EvalArgs a{d_y, on_dev ? targets : d_t, d_loss, d_pred, d_hit, n, width, loss_func,
                net->act[net->layers - 2] == A_SIGMOID ? 1 : 0};
     sp_eval_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(a);
@@ -1551,7 +1677,7 @@ static int time_common(sphip_net *const *nets, int count, const float *d_x, uint
     HCHECK(hipEventCreate(&e1));
     int rc = 0;
     HCHECK(hipEventRecord(e0, g_stream));
-    for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward(nets[it % count], d_x, n, d_y, flags, only_layer);
+    for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward(nets[it % count], nets[it % count]->workspace(), d_x, n, d_y, flags, only_layer);
     hipError_t e = hipEventRecord(e1, g_stream);
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
@@ -1594,7 +1720,7 @@ const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, 
     const float *aligned_ptr = reinterpret_cast<const float *>(uintptr_t{256});     // never dereferenced
     switch (pick_regime(net, n, flags)) {
     case R_GEMV:
-        launch_gemv(net, L, aligned_ptr, nullptr, n, false);
+        launch_gemv(net->prec, net->workspace(), L, aligned_ptr, nullptr, n, false);
         break;
     case R_GEMM32:
         (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
