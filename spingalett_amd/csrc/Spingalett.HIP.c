@@ -101,8 +101,8 @@ static sp_net *checked(NeuralNetwork *net, const char *who)
         sp_set_error(SPINGALETT_ERR_INVALID, "net is NULL");
         return NULL;
     }
-    sp_net *sn = sp_priv(net);
-    if (sn->magic != SP_NET_MAGIC) {
+    sp_net *sn = sp_owned(net);
+    if (!sn) {
         char msg[SP_ERRMSG_MAX];
         snprintf(msg, sizeof msg, "%s: network was not created by this library", who);
         sp_set_error(SPINGALETT_ERR_INVALID, msg);
@@ -197,8 +197,8 @@ void spingalett_hip_invalidate(NeuralNetwork *net)
 
 PrecisionMode spingalett_hip_precision(const NeuralNetwork *net)
 {
-    const sp_net *sn = (const sp_net *)(const void *)net;
-    if (!net || sn->magic != SP_NET_MAGIC) return PRECISION_FLOAT32;
+    const sp_net *sn = sp_owned(net);
+    if (!sn) return PRECISION_FLOAT32;
     if (sn->dev) return sn->dev_precision;
     return (sn->packed_w && sn->packed_b) ? sn->packed_precision : PRECISION_FLOAT32;
 }
@@ -244,6 +244,7 @@ static inline bool should_report(size_t epoch, size_t epochs, size_t interval)  
 static bool train_download(sp_net *sn)
 {
     NeuralNetwork *net = &sn->pub;
+    sn->opt_loaded = true;            /* the host gradient / moment arrays hold content from here on: layer() carries them */
     for (uint32_t l = 0; l + 1 < net->layers; ++l) {
         const uint64_t wo = net->weight_offsets[l], bo = net->bias_offsets[l];
         if (sphip_train_get(sn->dev, SPHIP_TRAIN_W, l, net->weights + wo) || sphip_train_get(sn->dev, SPHIP_TRAIN_B, l, net->biases + bo) ||

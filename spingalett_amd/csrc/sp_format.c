@@ -291,7 +291,7 @@ static NeuralNetwork *load_from_blob(uint8_t *blob, size_t bytes, const char *la
         return NULL;
     }
     net->time_step = time_step;
-    sp_net *sn = sp_priv(net);
+    sp_net *sn = sp_owned(net);           /* sp_net_build() just made it */
     sn->packed_w = (sp_packed_array *)calloc(layers - 1, sizeof(sp_packed_array));
     sn->packed_b = (sp_packed_array *)calloc(layers - 1, sizeof(sp_packed_array));
     if (!sn->packed_w || !sn->packed_b) {

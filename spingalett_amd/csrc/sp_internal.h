@@ -30,13 +30,17 @@ typedef struct {
     PrecisionMode    packed_precision;
     sp_packed_array *packed_w;      /* [layers-1] */
     sp_packed_array *packed_b;      /* [layers-1] */
-    bool             opt_loaded;    /* a file's optimizer block was read into opt_m/opt_v */
+    bool             opt_loaded;    /* opt_m / opt_v / grad_* may hold content: a file's optimizer block was read
+                                       into them, or train() copied the device's gradients and moments back */
     /* device side */
     sphip_net       *dev;
     PrecisionMode    dev_precision;
 } sp_net;
 
-static inline sp_net *sp_priv(NeuralNetwork *net) { return (sp_net *)(void *)net; }
+/* The private record of a net this library allocated and has not freed, else NULL.  Nothing past the
+ * public part of a caller's NeuralNetwork is read before the pointer has been found in the library's own
+ * table of live nets (sp_network.c). */
+sp_net *sp_owned(const NeuralNetwork *net);
 
 /* sp_runtime.c */
 void  sp_set_error(int code, const char *msg);

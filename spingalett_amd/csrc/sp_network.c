@@ -7,6 +7,7 @@
 #include "sp_internal.h"
 
 #include <math.h>
+#include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
 #include <time.h>
@@ -112,6 +113,44 @@ void print_parameters(NeuralNetwork *net)
     sp_log(LOG_INFO, "================================================");
 }
 
+/* ---- table of live nets ---- */
+static pthread_mutex_t g_live_mu = PTHREAD_MUTEX_INITIALIZER;
+static sp_net **g_live = NULL;
+static size_t g_live_n = 0, g_live_cap = 0;
+
+static bool live_add(sp_net *sn)
+{
+    bool ok = true;
+    pthread_mutex_lock(&g_live_mu);
+    if (g_live_n == g_live_cap) {
+        const size_t cap = g_live_cap ? 2 * g_live_cap : 16;
+        sp_net **t = (sp_net **)realloc(g_live, cap * sizeof *t);
+        if (t) { g_live = t; g_live_cap = cap; } else ok = false;
+    }
+    if (ok) g_live[g_live_n++] = sn;
+    pthread_mutex_unlock(&g_live_mu);
+    return ok;
+}
+
+static void live_remove(sp_net *sn)
+{
+    pthread_mutex_lock(&g_live_mu);
+    for (size_t i = 0; i < g_live_n; ++i)
+        if (g_live[i] == sn) { g_live[i] = g_live[--g_live_n]; break; }
+    pthread_mutex_unlock(&g_live_mu);
+}
+
+sp_net *sp_owned(const NeuralNetwork *net)
+{
+    sp_net *found = NULL;
+    if (!net) return NULL;
+    pthread_mutex_lock(&g_live_mu);
+    for (size_t i = 0; i < g_live_n; ++i)
+        if ((const void *)g_live[i] == (const void *)net) { found = g_live[i]; break; }
+    pthread_mutex_unlock(&g_live_mu);
+    return (found && found->magic == SP_NET_MAGIC) ? found : NULL;
+}
+
 /* ---- new_spingalett (Network.c:34-45) ---- */
 NeuralNetwork *new_spingalett_struct_arguments(NeuralNetworkArgs args)
 {
@@ -127,6 +166,11 @@ NeuralNetwork *new_spingalett_struct_arguments(NeuralNetworkArgs args)
     }
     sn->magic = SP_NET_MAGIC;
     sn->pub.loss_func = args.loss_func;
+    if (!live_add(sn)) {
+        free(sn);
+        sp_set_error(SPINGALETT_ERR_ALLOC, "NeuralNetwork calloc failed");
+        return NULL;
+    }
     return &sn->pub;
 }
 
@@ -141,9 +185,9 @@ static bool regrow(float **arr, uint64_t old_count, uint64_t new_count)
     return true;
 }
 
-/* Gradient / optimizer arrays are never written by this library: growing them
- * means a fresh zero block (the old contents are zero too unless a file with an
- * optimizer block was loaded, in which case they are carried over). */
+/* Gradient / optimizer arrays: while nothing has written them (no optimizer block loaded, no
+ * train() call) they are all zero, and growing them means a fresh zero block instead of a copy;
+ * with `carry` the old contents move over like the weights do. */
 static bool regrow_lazy(float **arr, uint64_t old_count, uint64_t new_count, bool carry)
 {
     if (carry) return regrow(arr, old_count, new_count);
@@ -162,7 +206,7 @@ void layer_struct_arguments(LayerArgs args)
         sp_set_error(SPINGALETT_ERR_INVALID, "Net is NULL or neurons amount is 0");
         return;
     }
-    sp_net *sn = sp_priv(net);
+    sp_net *sn = sp_owned(net);           /* NULL for a record the caller made up: no device state, nothing loaded */
     const uint32_t old_layers = net->layers, nl = old_layers + 1;
     if (nl > 1) {
         if ((unsigned)args.act_func >= ACT_COUNT) {
@@ -201,10 +245,12 @@ void layer_struct_arguments(LayerArgs args)
     }
     ok = ok && regrow(&net->neurons, net->total_neurons, tn);
     if (ok && nl > 1) {
-        const bool carry = sn->magic == SP_NET_MAGIC && sn->opt_loaded;   /* only a loaded optimizer block has content */
+        /* gradients and moments are carried over like the weights (Network.c:130-146) whenever they can hold
+           anything: after a file's optimizer block was loaded or train() ran; otherwise they are still zero */
+        const bool carry = !sn || sn->opt_loaded;
         ok = regrow(&net->weights, net->total_weights, tw) && regrow(&net->biases, net->total_biases, tb)
-          && regrow_lazy(&net->grad_weights, net->total_weights, tw, false)
-          && regrow_lazy(&net->grad_biases, net->total_biases, tb, false)
+          && regrow_lazy(&net->grad_weights, net->total_weights, tw, carry)
+          && regrow_lazy(&net->grad_biases, net->total_biases, tb, carry)
           && regrow_lazy(&net->opt_m_weights, net->total_weights, tw, carry)
           && regrow_lazy(&net->opt_m_biases, net->total_biases, tb, carry)
           && regrow_lazy(&net->opt_v_weights, net->total_weights, tw, carry)
@@ -247,7 +293,7 @@ void layer_struct_arguments(LayerArgs args)
     net->total_biases = b;
 
     /* shape changed: whatever the device or a loaded file held is stale */
-    if (sn->magic == SP_NET_MAGIC) {
+    if (sn) {
         sp_hip_release(sn);
         sp_drop_packed(sn);
     }
@@ -262,6 +308,10 @@ NeuralNetwork *sp_net_build(LossFunction loss, uint32_t layers, const uint32_t *
     sp_net *sn = (sp_net *)calloc(1, sizeof *sn);
     if (!sn) return NULL;
     sn->magic = SP_NET_MAGIC;
+    if (!live_add(sn)) {
+        free(sn);
+        return NULL;
+    }
     NeuralNetwork *net = &sn->pub;
     net->loss_func = loss;
     net->layers = layers;
@@ -318,8 +368,8 @@ float *forward_struct_arguments(ForwardArgs args)
         sp_set_error(SPINGALETT_ERR_INVALID, "Network must have at least 2 layers for forward pass");
         return NULL;
     }
-    sp_net *sn = sp_priv(net);
-    if (sn->magic != SP_NET_MAGIC) {
+    sp_net *sn = sp_owned(net);
+    if (!sn) {
         sp_set_error(SPINGALETT_ERR_INVALID, "forward: network was not created by this library");
         return NULL;
     }
@@ -330,10 +380,11 @@ float *forward_struct_arguments(ForwardArgs args)
 void free_network(NeuralNetwork *net)
 {
     if (!net) return;
-    sp_net *sn = sp_priv(net);
-    if (sn->magic == SP_NET_MAGIC) {
+    sp_net *sn = sp_owned(net);
+    if (sn) {
         sp_hip_release(sn);
         sp_drop_packed(sn);
+        live_remove(sn);
         sn->magic = 0;
     }
     sp_aligned_free(net->neurons);

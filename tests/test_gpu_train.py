@@ -268,6 +268,33 @@ def test_small_batch_train_learns_xor_and_counts_steps():
     S.free_network(net)
 
 
+def test_layer_after_train_keeps_gradients_and_moments():
+    """layer() copies all six gradient / moment arrays into the regrown net (Network.c:130-146): adding a head after
+    train() (fine-tuning) must not zero what train() left in the host arrays."""
+    net, _ = public_net([2, 8, 3], ["tanh", "sigmoid"], 0, seed=5)
+    X = np.float32([[0, 0], [0, 1], [1, 0], [1, 1]] * 4)
+    T = np.float32([[0, 1, 0], [1, 0, 1], [1, 1, 0], [0, 0, 1]] * 4)
+    S.clear_error()
+    S.train(net, X, T, 5, S.STRATEGY_FULL_BATCH, S.OPTIMIZER_ADAM, learning_rate=0.05)
+    assert S.last_error()[0] == S.SPINGALETT_OK, S.last_error()
+    nc = net.contents
+    tw, tb = int(nc.total_weights), int(nc.total_biases)
+    view = lambda name, cnt: np.ctypeslib.as_array(getattr(net.contents, name), shape=(cnt,)).copy()
+    names_w = ["weights", "grad_weights", "opt_m_weights", "opt_v_weights"]
+    names_b = ["biases", "grad_biases", "opt_m_biases", "opt_v_biases"]
+    before = {k: view(k, tw) for k in names_w} | {k: view(k, tb) for k in names_b}
+    assert all(np.any(before[k] != 0) for k in before)              # train() really left something in every one
+    steps = nc.time_step
+    S.layer(net, 4, S.ACT_NONE, S.WEIGHT_INITIALIZATION_XAVIER)
+    assert net.contents.time_step == steps
+    for k in names_w:
+        assert np.array_equal(view(k, tw), before[k]), k            # old prefix unchanged
+    for k in names_b:
+        assert np.array_equal(view(k, tb), before[k]), k
+    assert not view("opt_m_weights", tw + 12)[tw:].any() and not view("grad_biases", tb + 4)[tb:].any()   # new part zero
+    S.free_network(net)
+
+
 def test_callback_stops_training_and_autosave_writes_files(tmp_path):
     net, _ = public_net([4, 6, 2], ["relu", "none"], 0)
     rng = np.random.default_rng(0)

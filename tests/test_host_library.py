@@ -296,6 +296,32 @@ def test_settings_and_error_slot(S):
     assert S.last_error() == (0, "")
 
 
+def test_a_record_the_library_did_not_allocate_is_recognised(S):
+    """The private state lives behind the public record, so the library looks a caller's pointer up in its own
+    table of live nets before reading past the public part: a NeuralNetwork made up by the caller (exactly as
+    large as the public struct) is refused by forward() and reports FP32, a freed-and-recreated one is fine."""
+    import ctypes as C
+    fake = S.NeuralNetwork()
+    fake.layers = 2
+    x = np.zeros(4, np.float32)
+    S.clear_error()
+    out = S.lib().forward_struct_arguments(S.ForwardArgs(C.pointer(fake), x.ctypes.data_as(C.POINTER(C.c_float))))
+    assert not out
+    code, msg = S.last_error()
+    assert code == S.SPINGALETT_ERR_INVALID and "not created by this library" in msg
+    S.clear_error()
+    assert S.lib().spingalett_hip_precision(C.pointer(fake)) == S.PRECISION_FLOAT32
+    S.lib().spingalett_hip_invalidate(C.pointer(fake))
+    assert S.last_error()[0] == S.SPINGALETT_ERR_INVALID
+    S.clear_error()
+    for _ in range(40):                                  # the table grows and shrinks
+        nets = [S.new_spingalett() for _ in range(5)]
+        for n in nets:
+            S.layer(n, 3)
+            S.free_network(n)
+    assert S.last_error()[0] == S.SPINGALETT_OK
+
+
 def test_forward_fails_loudly_without_a_gpu(S):
     if S.device_count() > 0:
         pytest.skip("a GPU is present")

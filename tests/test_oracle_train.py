@@ -243,6 +243,62 @@ def test_rmsprop_per_sample_rule_folds_decay_into_the_gradient():
     np.testing.assert_allclose(n1.weights, n2.weights, rtol=1e-6)
 
 
+@pytest.mark.parametrize("opt", [O.OPT_ADAM, O.OPT_ADAMW])
+@pytest.mark.parametrize("b1,b2", [(0.9, 0.999), (0.5, 0.7)])
+def test_adam_moment_recurrences_under_a_constant_gradient(opt, b1, b2):
+    """Steps 1..5 with the same gradient (SIMD.c:279-382): m_t = (1 - b1^t) g and v_t = (1 - b2^t) g^2, so the
+    bias-corrected moments stay g and g^2 and every step moves a weight by lr g / sqrt(g^2 + eps); AdamW
+    shrinks the weight by (1 - lr wd) before each of them.  A wrong coefficient on the beta m / beta v terms,
+    which a first step from zero moments cannot see, breaks the moments from step 2 on."""
+    lr, eps, wd = 0.01, 1e-8, (0.3 if opt == O.OPT_ADAMW else 0.0)
+    net, st, gW, gB = _fresh()
+    w = net.weights.astype(np.float64)
+    b = net.biases.astype(np.float64)
+    g64, gb64 = gW.astype(np.float64), gB.astype(np.float64)
+    omb1, omb2 = float(np.float32(1) - np.float32(b1)), float(np.float32(1) - np.float32(b2))
+    for t in range(1, 6):
+        net.apply_gradients(st, gW.copy(), gB.copy(), opt, lr=lr, beta1=b1, beta2=b2, epsilon=eps, weight_decay=wd)
+        w = w * (1 - lr * wd) - lr * g64 / np.sqrt(g64 ** 2 + eps)
+        b = b - lr * gb64 / np.sqrt(gb64 ** 2 + eps)                        # biases are never decayed
+        np.testing.assert_allclose(net.weights, w, rtol=5e-5, atol=2e-7, err_msg=f"step {t}")
+        np.testing.assert_allclose(net.biases, b, rtol=5e-5, atol=2e-7, err_msg=f"step {t}")
+        # geometric sums of the recurrences, with 1 - beta as the reference forms it in FP32
+        np.testing.assert_allclose(st.mW, omb1 * g64 * sum(b1 ** k for k in range(t)), rtol=2e-5, err_msg=f"m, step {t}")
+        np.testing.assert_allclose(st.vW, omb2 * g64 ** 2 * sum(b2 ** k for k in range(t)), rtol=2e-5, err_msg=f"v, step {t}")
+        assert float(st.beta1_pow) == pytest.approx(b1 ** t, rel=1e-5) and float(st.beta2_pow) == pytest.approx(b2 ** t, rel=1e-5)
+
+
+def test_adam_second_step_with_a_doubled_gradient():
+    """g then 2 g: m_2 = (1 - b1)(b1 + 2) g and v_2 = (1 - b2)(b2 + 4) g^2, corrected by 1 - b^2: the two betas
+    enter with different weights, so exchanging them (or their moments) shows."""
+    lr, eps, b1, b2 = 0.01, 1e-8, 0.6, 0.9
+    net, st, gW, gB = _fresh()
+    w0 = net.weights.astype(np.float64)
+    g = gW.astype(np.float64)
+    net.apply_gradients(st, gW.copy(), gB.copy(), O.OPT_ADAM, lr=lr, beta1=b1, beta2=b2, epsilon=eps)
+    net.apply_gradients(st, 2 * gW, 2 * gB, O.OPT_ADAM, lr=lr, beta1=b1, beta2=b2, epsilon=eps)
+    m2 = (1 - b1) * (b1 + 2) * g / (1 - b1 ** 2)
+    v2 = (1 - b2) * (b2 + 4) * g ** 2 / (1 - b2 ** 2)
+    want = w0 - lr * g / np.sqrt(g ** 2 + eps) - lr * m2 / np.sqrt(v2 + eps)
+    np.testing.assert_allclose(net.weights, want, rtol=5e-5, atol=2e-7)
+
+
+def test_rmsprop_second_moment_recurrence_under_a_constant_gradient():
+    """SIMD.c:455-494: v_t = (1 - b2^t) g^2 (no bias correction), so step t moves a weight by
+    lr g / sqrt((1 - b2^t) g^2 + eps)."""
+    lr, b2, eps = 0.02, 0.8, 1e-6
+    net, st, gW, gB = _fresh()
+    w = net.weights.astype(np.float64)
+    g = gW.astype(np.float64)
+    omb2 = float(np.float32(1) - np.float32(b2))
+    for t in range(1, 6):
+        net.apply_gradients(st, gW.copy(), gB.copy(), O.OPT_RMSPROP, lr=lr, beta2=b2, epsilon=eps)
+        vt = omb2 * g ** 2 * sum(b2 ** k for k in range(t))
+        w = w - lr * g / np.sqrt(vt + eps)
+        np.testing.assert_allclose(st.vW, vt, rtol=2e-5, err_msg=f"v, step {t}")
+        np.testing.assert_allclose(net.weights, w, rtol=5e-5, atol=2e-7, err_msg=f"step {t}")
+
+
 def test_clipping_precedes_the_update():
     net, st, gW, gB = _fresh()
     w0 = net.weights.copy()
