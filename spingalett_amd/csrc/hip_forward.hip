@@ -246,6 +246,18 @@ __device__ __forceinline__ uint16_t f32_to_t16(float x)
     else return f32_to_bf16_rne(x);
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 __device__ __forceinline__ float wave_sum(float v)
 {
 #pragma unroll
@@ -690,6 +702,33 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
     a.meta_bytes = a.nchunks * n * 16u;
     if ((uint64_t)kc_blocks * blk_bytes + a.meta_bytes > 156u * 1024u) return false;
     const uint32_t nblocks = a.nchunks * kc_blocks;
+    a.rw = rw;
+    a.ks = ks;
+    const uint32_t waves = rw * ks;
+    const uint32_t grid = (wave_rows + rw - 1) / rw;
+    const size_t red_bytes = (size_t)waves * MT * 64u * sizeof(float);
+    tl_route.name = "sp_gemv_i8mfma";
+    if (fused) {
+        // digit planes in LDS: all of K in one buffer if that takes at most 120 KB, else two buffers of whole scale
+        // chunks (at most 60 KB each) that the quant waves fill in turn
+        uint32_t stage = nblocks;
+        size_t lds = (size_t)nblocks * blk_bytes;
+        if (lds > 120u * 1024u) {
+            stage = (60u * 1024u / blk_bytes) / kc_blocks * kc_blocks;
+            if (stage == 0) stage = kc_blocks;
+            lds = 2u * (size_t)stage * blk_bytes;
+        }
+        a.stage_blocks = stage;
+        if (lds < red_bytes) lds = red_bytes;
+        lds += a.meta_bytes;
+        // one quant wave per (scale chunk, sample) of the first stage, at most eight
+        const uint32_t units = (stage / kc_blocks < a.nchunks ? stage / kc_blocks : a.nchunks) * n;
+        a.qw = units < 8u ? units : 8u;
+        // how a K share's blocks are chosen: see gemv_i8_specialised
+        if ((uint64_t)L.N * L.K * I8Fmt<FMT>::bits / 8u > (64ull << 20)) launch_gemv_i8_mt<FMT, 1, 2>(a, grid, (waves + a.qw) * 64, lds);
+        else launch_gemv_i8_mt<FMT, 1, 1>(a, grid, (waves + a.qw) * 64, lds);
+        return true;
+    }
     // LDS stage: everything if it fits the budget, else whole scale chunks
     uint32_t stage = nblocks;
     if ((uint64_t)nblocks * blk_bytes > budget) {
@@ -697,25 +736,9 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
         if (stage == 0) stage = kc_blocks;
     }
     a.stage_blocks = stage;
-    a.rw = rw;
-    a.ks = ks;
-    const uint32_t waves = rw * ks;
-    const uint32_t grid = (wave_rows + rw - 1) / rw;
     size_t lds = (size_t)stage * blk_bytes;
-    const size_t red_bytes = (size_t)waves * MT * 64u * sizeof(float);
     if (lds < red_bytes) lds = red_bytes;
     lds += a.meta_bytes;
-    tl_route.name = "sp_gemv_i8mfma";
-    if (fused) {
-        // samples one wave quantises at once: as many as still leave every wave a unit of work
-        const uint32_t cps = stage / kc_blocks;
-        uint32_t ns = 4;
-        while (ns > 1 && (ns / 2 >= n || cps * ((n + ns - 1) / ns) < waves)) ns >>= 1;
-        if (ns == 1) launch_gemv_i8_mt<FMT, 1, 1>(a, grid, waves * 64, lds);
-        else if (ns == 2) launch_gemv_i8_mt<FMT, 1, 2>(a, grid, waves * 64, lds);
-        else launch_gemv_i8_mt<FMT, 1, 4>(a, grid, waves * 64, lds);
-        return true;
-    }
     if (!main_only && !tl_route.dry) sp_quant_x<FMT><<<(a.nchunks * n + 3u) / 4u, 256, 0, g_stream>>>(a);
     switch (MT) {
     case 1:  launch_gemv_i8_mt<FMT, 1>(a, grid, waves * 64, lds); break;
@@ -959,6 +982,12 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
             static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
             (void)once;
             kern<<<grid, 512, lds, g_stream>>>(g);
+        } else if (getenv("SPHIP_GEMM_VARIANT") && atoi(getenv("SPHIP_GEMM_VARIANT")) == 4) {
+            constexpr size_t lds = 2 * (256 + 256) * 64 * sizeof(uint16_t);
+            auto kern = sp_gemm16_big<FMT, F16T, 2, 2, 4, 4>;
+            static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            kern<<<grid, 256, lds, g_stream>>>(g);
         } else {
             constexpr size_t lds = 2 * (256 + 256) * 64 * sizeof(uint16_t);
             auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;

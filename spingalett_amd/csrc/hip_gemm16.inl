@@ -312,18 +312,6 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     }
 }
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
-template <int N, int I = 0, class F>
-__device__ __forceinline__ void static_for(F &&f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<N, I + 1>(f);
-    }
-}
-
 template <int OFF>
 __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
 
@@ -424,12 +412,14 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     // Only the first wave of each SIMD (waves 0 .. NWAVES/2-1, which the issue arbiter serves first)
     // issues the loads, for itself and for wave + NWAVES/2: a wave stalls while the address unit takes
     // its load, and the other wave of the SIMD keeps the MFMA pipe fed meanwhile.
-    constexpr int HALF = NWAVES / 2;
-    constexpr int A_DUTY = 2 * A_ISSUES, W_DUTY = W_DIRECT ? 2 * W_ISSUES : 1;
+    // (four-wave workgroups have one wave per SIMD: every wave loads its own share)
+    constexpr int HALF = NWAVES > 4 ? NWAVES / 2 : NWAVES;      // loader waves
+    constexpr int PER = NWAVES / HALF;                            // shares a loader wave issues
+    constexpr int A_DUTY = PER * A_ISSUES, W_DUTY = W_DIRECT ? PER * W_ISSUES : 1;
     uint32_t a_voff[A_DUTY], w_voff[W_DUTY];
 #pragma unroll
     for (int d = 0; d < A_DUTY; ++d) {
-        const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+        const int i = d / PER, wv = (wave & (HALF - 1)) + (d % PER) * HALF;
         const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
         const uint32_t m = m0 + row < M ? m0 + row : M - 1;
         a_voff[d] = (uint32_t)(((size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
@@ -437,7 +427,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     if constexpr (W_DIRECT) {
 #pragma unroll
         for (int d = 0; d < W_DUTY; ++d) {
-            const int i = d >> 1, wv = (wave & (HALF - 1)) + (d & 1) * HALF;
+            const int i = d / PER, wv = (wave & (HALF - 1)) + (d % PER) * HALF;
             const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
             const uint32_t n = n0 + row < N ? n0 + row : N - 1;
             w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
@@ -458,13 +448,13 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 #pragma unroll
         for (int d = 0; d < A_DUTY; ++d)
             if (d == idx)
-                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), a_voff[d],
+                lds_dma16(lds_a + (uint32_t)(buf * BM * BK * 2 + ((d / PER) * NWAVES + (d % PER) * HALF) * 1024), a_voff[d],
                           a_base + (size_t)k0 * 2u);
         if constexpr (W_DIRECT) {
 #pragma unroll
             for (int d = 0; d < W_DUTY; ++d)
                 if (A_DUTY + d == idx)
-                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d >> 1) * NWAVES + (d & 1) * HALF) * 1024), w_voff[d],
+                    lds_dma16(lds_w + (uint32_t)(buf * BN * BK * 2 + ((d / PER) * NWAVES + (d % PER) * HALF) * 1024), w_voff[d],
                               w_base + (size_t)k0 * 2u);
         }
     };

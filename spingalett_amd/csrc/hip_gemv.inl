@@ -191,7 +191,8 @@ struct GemvI8Args {
     uint32_t kc;           // K chunk = one scale block (multiple of the 64-byte block)
     uint32_t nchunks;      // ceil(K / kc)
     uint32_t stage_blocks; // 64-byte blocks whose digit planes are held in LDS at a time
-    uint32_t rw, ks;       // waves of a workgroup: row groups x K shares
+    uint32_t rw, ks;       // waves of a workgroup that multiply: row groups x K shares
+    uint32_t qw;           // self-quantising form: waves of a workgroup that quantise the activations (after the rw x ks others)
     uint32_t meta_bytes;   // LDS bytes of the per-chunk scale records (multiple of 16)
 };
 
@@ -254,7 +255,6 @@ struct QuantRegs {
     static constexpr int MAXIT = 2048 / (64 * I8Fmt<FMT>::WK);
     static constexpr int F4 = I8Fmt<FMT>::WK / 4;
     float4 v[NS][MAXIT][F4];
-    uint32_t m[NS];      // largest |x| as its bit pattern: orders like the value, and infinities and NaNs sort last
 };
 
 template <int FMT, int NS>
@@ -267,7 +267,6 @@ __device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *x
     const uint32_t iters = kc / (64u * WK);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        q.m[s] = 0u;
         const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
@@ -281,9 +280,6 @@ __device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *x
                 float4 t = src[c];
                 if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 q.v[s][it][c] = t;
-                const uint32_t mx = max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu);
-                const uint32_t mz = max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu);
-                q.m[s] = max(q.m[s], max(mx, mz));
             }
         }
     }
@@ -299,7 +295,18 @@ __device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
         if (s >= ns) break;
-        const uint32_t amax = wave_max_u(q.m[s]);
+        // largest |x| of the chunk as its bit pattern: orders like the value, and infinities and NaNs sort last
+        uint32_t lm = 0u;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it)
+#pragma unroll
+            for (int c = 0; c < F::WK / 4; ++c) {
+                const float4 t = q.v[s][it][c];
+                const uint32_t mx = max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu);
+                const uint32_t mz = max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu);
+                lm = max(lm, max(mx, mz));
+            }
+        const uint32_t amax = wave_max_u(lm);
         int e = (int)(amax >> 23) - 127;
         if (e < -126) e = -126;
         int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
@@ -361,6 +368,252 @@ __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
         });
 }
 
+// Self-quantising form for up to four samples: one launch per layer, the waves of a workgroup specialised.
+//   * Quant waves (the qw waves after the stream waves) request the activations of their first scale chunk before
+//     anything else in the workgroup touches memory, and only when those have arrived are the stream waves let go
+//     (barrier "go"): a compute unit's memory pipeline returns data in request order, and activations queued behind
+//     megabytes of weight requests arrived 1.3 us later per fetch group in flight.  They then quantise into LDS, one
+//     scale chunk of one sample at a time, and meet the stream waves at barrier 0.
+//   * Stream waves (rw row groups x ks K shares; wave = ks_id * rw + rw_id) request D fetch groups of G 64-byte blocks
+//     of their 16 rows, wait at barrier 0 for the digit planes, then multiply group by group; a group's registers are
+//     reloaded with the group D further on as soon as it has been multiplied (D register sets, rotated by unrolling:
+//     no copies, and the counted wait before a group leaves the younger requests in flight).  The weight stream so
+//     runs while the activations are quantised (about 1.5 us during which memory used to sit idle).
+//   * Which blocks a K share takes (PAIRS): pairs of blocks ks_id, ks_id + ks, ... (whole 128-byte lines per wave;
+//     with three groups of one pair in flight the better choice up to 64 MiB of weights: 8192 x 8192 INT8 17.1
+//     against 18.2 us, INT2 8.9 against 9.6 us, 4096 x 16384 INT4 11.5 against 13.3 us) or single blocks ks_id,
+//     ks_id + ks, ... (two groups of four blocks; the halves of a line then come from two waves at about the same
+//     time, which the memory system serves faster on large layers: 16384 x 16384 INT4 30.2 against 31.8 us, INT8 56
+//     against 64 us).  Deeper prefetch than these was measured and is slower in either form.
+// Digit planes of more than one LDS buffer (a.stage_blocks) take two buffers, stage s in buffer s & 1: the quant
+// waves fill stage s + 1 while stage s is multiplied, and barrier s separates "stage s written" from "stage s read"
+// for every wave (a buffer is refilled only after the barrier that ends its reading).
+// 16 bytes per lane from a 64-bit lane address.  Inline assembly: the compiler's wait-count bookkeeping does not see
+// the load (it would wait for every outstanding one where only the oldest set is needed); the caller waits with
+// s_waitcnt vmcnt before it reads dst, and before the registers can be reused for anything else.
+__device__ __forceinline__ void gload16_async(u32x4 &dst, const void *p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+
+template <int FMT, int D, int G, bool PAIRS>
+__device__ __forceinline__ void gemv_i8_specialised(const GemvI8Args &a)
+{
+    using F = I8Fmt<FMT>;
+    constexpr int KL = F::KL, NMF = F::NMF;
+    static_assert(G == 2 || G == 4, "fetch groups of two or four blocks");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    int4 *meta = reinterpret_cast<int4 *>(lds_all);               // [nchunks][nb] {2^-p bits, d0 sum, d1 sum, d2 sum}
+    uint8_t *A_lds = lds_all + a.meta_bytes;                      // [2][stage blocks][NMF][4 g][nb][3][16 bytes]
+
+    const int t = threadIdx.x, lane = t & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t N = a.L.N, K = a.L.K;
+    const uint32_t nb = (uint32_t)a.nb;
+    const uint32_t rw = a.rw, ks = a.ks, sw = rw * ks;
+    const uint32_t kcb = a.kc / KL;                               // blocks per scale chunk
+    const uint32_t blk_bytes = (uint32_t)NMF * 4u * nb * 48u;     // digit planes of one block
+    const uint32_t u_bytes = 4u * nb * 48u;
+    const uint32_t cps = a.stage_blocks / kcb;                    // chunks per stage
+    const uint32_t nstages = (a.nchunks + cps - 1) / cps;
+    const uint32_t buf_bytes = a.stage_blocks * blk_bytes;
+
+    if (wave >= sw) {
+        // ---- quant wave
+        const uint32_t qid = wave - sw;
+        QuantRegs<FMT, 1> qr;
+        // The first unit's activations are requested before any weight and have arrived when the stream waves are let
+        // go (barrier "go"): the memory pipeline of a compute unit returns data in request order, and activations
+        // queued behind a few megabytes of weight requests arrive microseconds later.
+        {
+            const uint32_t nch0 = cps <= a.nchunks ? cps : a.nchunks;
+            if (qid < nch0 * nb) {
+                quant_load<FMT, 1>(qr, a.x + (size_t)(qid % nb) * K, K, (qid / nb) * a.kc, a.kc, 1, lane);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __syncthreads();                                      // barrier "go"
+        }
+        for (uint32_t s = 0; s < nstages; ++s) {
+            const uint32_t ch0 = s * cps, nch = ch0 + cps <= a.nchunks ? cps : a.nchunks - ch0;
+            uint8_t *buf = A_lds + (size_t)(s & 1u) * buf_bytes;
+            for (uint32_t ui = qid; ui < nch * nb; ui += a.qw) {
+                const uint32_t chl = ui / nb, smp = ui % nb;
+                if (s != 0 || ui != qid)                          // the first unit is in the registers already
+                    quant_load<FMT, 1>(qr, a.x + (size_t)smp * K, K, (ch0 + chl) * a.kc, a.kc, 1, lane);
+                quant_finish<FMT, 1>(qr, a.kc, 1, lane,
+                    [&](uint32_t, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+                        uint8_t *dst = buf + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + smp) * 48 + w * 4;
+                        *reinterpret_cast<uint32_t *>(dst) = d0;
+                        *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+                        *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+                    },
+                    [&](uint32_t, int4 md) {
+                        if (lane == 0) meta[(size_t)(ch0 + chl) * nb + smp] = md;
+                    });
+            }
+            __syncthreads();                                      // barrier s: stage s is written
+        }
+        if (ks > 1) {                                             // the two barriers of the K-share reduction
+            __syncthreads();
+            __syncthreads();
+        }
+        return;
+    }
+
+    // ---- stream wave
+    const uint32_t ks_id = wave / rw, rw_id = wave % rw;
+    const uint32_t nrow = (blockIdx.x * rw + rw_id) * 16u + (lane & 15);
+    const uint32_t g = lane >> 4;
+    const size_t row_bytes = (size_t)K * F::bits / 8u;
+    const uint8_t *wrow = a.L.w + (size_t)(nrow < N ? nrow : N - 1) * row_bytes + g * 16u;
+    // largest offset (from wrow) whose 16 bytes stay inside the row; reads past it are clamped there and meet zero digits
+    const int64_t row_last = (int64_t)row_bytes - 16 - (int64_t)(g * 16u);
+    const uint32_t groups_per_chunk = kcb / (ks * G);             // host guarantees divisibility
+    const uint32_t ngroups = a.nchunks * groups_per_chunk;
+
+    // Block u of this wave's fetch group j is block first + j * adv + du(u) of the row:
+    //   PAIRS: block (u & 1) of pair ((G / 2) j + (u >> 1)) * ks + ks_id;  else block (G j + u) * ks + ks_id
+    const uint32_t first = PAIRS ? 2u * ks_id : ks_id;
+    const uint32_t adv = (uint32_t)G * ks;
+    auto du = [&](int u) { return PAIRS ? (uint32_t)(u >> 1) * 2u * ks + (uint32_t)(u & 1) : (uint32_t)u * ks; };
+    auto load_group = [&](u32x4 (&dst)[G], uint32_t j) {
+#pragma unroll
+        for (int u = 0; u < G; ++u) {
+            int64_t off = (int64_t)((first + j * adv + du(u)) * 64u);
+            off = off < row_last ? off : row_last;
+            off = off > 0 ? off : 0;
+            gload16_async(dst[u], wrow + off);
+        }
+    };
+    __syncthreads();                                              // barrier "go": the quant waves hold their activations
+    u32x4 R[D][G];
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if ((uint32_t)d < ngroups) load_group(R[d], (uint32_t)d);
+
+    // lane (m, g): row m of the A tile is digit m & 3 of sample m >> 2 (fourth rows and samples beyond nb are never
+    // read from D: they point at the start of the block)
+    uint32_t a_off;
+    {
+        const uint32_t m = lane & 15u, slot = m >> 2, d = m & 3u;
+        a_off = (slot < nb && d < 3u) ? ((g * nb + slot) * 3u + d) * 16u : 0u;
+    }
+    float yacc = 0.0f;
+    i32x4v acc[2] = {(i32x4v){0, 0, 0, 0}, (i32x4v){0, 0, 0, 0}};
+
+    auto process = [&](const u32x4 wv, const uint8_t *rec) {
+        const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+        i32x4v bop[NMF];
+        if constexpr (FMT == I8) {
+            bop[0] = (i32x4v){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        } else if constexpr (FMT == I4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x8 = w[q] ^ 0x88888888u;          // nibble -> q + 8
+                bop[0][q] = (int)(x8 & 0x0F0F0F0Fu);
+                bop[1][q] = (int)((x8 >> 4) & 0x0F0F0F0Fu);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t x2 = w[q] ^ 0xAAAAAAAAu;          // field -> q + 2
+                bop[0][q] = (int)(x2 & 0x03030303u);
+                bop[1][q] = (int)((x2 >> 2) & 0x03030303u);
+                bop[2][q] = (int)((x2 >> 4) & 0x03030303u);
+                bop[3][q] = (int)((x2 >> 6) & 0x03030303u);
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < NMF; ++f) {
+            const i32x4v aop = *reinterpret_cast<const i32x4v *>(rec + f * u_bytes + a_off);
+            acc[f & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, bop[f], acc[f & 1], 0, 0, 0);
+        }
+    };
+    auto fold = [&](uint32_t ch) {
+        if (g < nb) {
+            const int4 md = meta[(size_t)ch * nb + g];
+            int S0 = acc[0][0] + acc[1][0], S1 = acc[0][1] + acc[1][1], S2 = acc[0][2] + acc[1][2];
+            if (F::BIAS != 0 && ks_id == 0) {           // one K share removes the code bias of the whole chunk
+                S0 -= F::BIAS * md.y;
+                S1 -= F::BIAS * md.z;
+                S2 -= F::BIAS * md.w;
+            }
+            const float tsum = fmaf((float)S2, 65536.0f, fmaf((float)S1, 256.0f, (float)S0));
+            yacc = fmaf(tsum, __int_as_float(md.x), yacc);
+        }
+        acc[0] = acc[1] = (i32x4v){0, 0, 0, 0};
+    };
+
+    __syncthreads();                                              // barrier 0
+    const uint8_t *rec = A_lds + (size_t)first * blk_bytes;       // digit planes of the first block of the current group
+    uint32_t jnext = (uint32_t)D;                                 // next fetch group to request
+    uint32_t gi = 0, ch = 0, cis = 0, stage = 0;
+    // waits until at most `groups` fetch groups are outstanding (a uniform choice among the constants the
+    // instruction can carry)
+    auto wait_groups = [&](uint32_t groups) {
+        static_for<D>([&](auto yc) {
+            constexpr int y = decltype(yc)::value;
+            if (groups == (uint32_t)y) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(y * G) : "memory");
+        });
+    };
+    uint32_t jcur = 0;                                            // fetch group about to be multiplied
+    auto step = [&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        // this set's requests are the oldest outstanding; younger ones: the groups requested after it, at most D - 1
+        // and fewer near the end of the row, where nothing is requested any more
+        const uint32_t younger = ngroups - 1u - jcur;
+        wait_groups(younger < (uint32_t)(D - 1) ? younger : (uint32_t)(D - 1));
+#pragma unroll
+        for (int u = 0; u < G; ++u) asm volatile("" : "+v"(R[d][u]));      // nothing that reads them moves above the wait
+#pragma unroll
+        for (int u = 0; u < G; ++u) process(R[d][u], rec + (size_t)du(u) * blk_bytes);
+        if (jnext < ngroups) load_group(R[d], jnext);
+        ++jnext;
+        ++jcur;
+        rec += (size_t)adv * blk_bytes;
+        if (++gi == groups_per_chunk) {
+            gi = 0;
+            fold(ch);
+            ++ch;
+            if (++cis == cps && ch < a.nchunks) {                 // next stage: the other buffer, once it is written
+                cis = 0;
+                ++stage;
+                __syncthreads();
+                rec = A_lds + (size_t)(stage & 1u) * buf_bytes + (size_t)first * blk_bytes;
+            }
+        }
+    };
+    for (uint32_t gdone = 0; gdone < ngroups; gdone += D) {
+        static_for<D>([&](auto dc) {
+            if (gdone + (uint32_t)decltype(dc)::value < ngroups) step(dc);
+        });
+    }
+
+    // add the K shares of a row group (in share order) through LDS
+    if (ks > 1) {
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(A_lds);             // [ks][rw][64]
+        if (ks_id > 0) red[((size_t)ks_id * rw + rw_id) * 64 + lane] = yacc;
+        __syncthreads();
+        if (ks_id > 0) return;
+        for (uint32_t o = 1; o < ks; ++o) yacc += red[((size_t)o * rw + rw_id) * 64 + lane];
+    }
+    if (nrow < N && g < nb) {
+        const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, nrow) * a.L.bscale;
+        float dot = yacc;
+        if (dot != dot) {
+            // the sample's input holds an infinity or a NaN (the integer sums themselves are always finite):
+            // plain FP32 multiply-adds over the row, in k order
+            const float *xs = a.x + (size_t)g * K;
+            const uint64_t base = (uint64_t)nrow * K;
+            dot = 0.0f;
+            for (uint32_t k = 0; k < K; ++k) dot = fmaf((float)int_code<FMT>(a.L.w, base + k), xs[k], dot);
+        }
+        a.y[(size_t)g * N + nrow] = apply_act(fmaf(dot, a.L.wscale, bias), a.L.act);
+    }
+}
+
+// Two-launch form (planes prepared by sp_quant_x; more than four samples, reachable with SPHIP_FORCE_GEMV).
 // MT = 16-row A tiles (four samples each).  Rows of D that belong to no sample
 // (fourth row of a slot, slots beyond nb) are never read, so their lanes may load
 // anything: they are pointed at the start of the block.
@@ -369,12 +622,16 @@ __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
 // Weights are fetched in groups of four blocks, the next group in flight while
 // the current one is multiplied; scale chunks are whole numbers of groups.
 //
-// FQ > 0 (n <= FQ <= 4): the workgroup (at most 8 waves) quantises the activations itself,
-// straight into LDS, instead of copying planes a separate launch prepared: every workgroup
-// repeats the (small) job, and the layer costs one launch instead of two.
+// FQ = 1, 2 select the self-quantising form above instead (one launch per layer; 1: K shares of whole lines, 2: of blocks).
 template <int FMT, int MT, int FQ>
-__global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
+__global__ __launch_bounds__(FQ ? 1024 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfma(const GemvI8Args a)
 {
+    if constexpr (FQ != 0) {
+        static_assert(FQ == 0 || MT == 1, "the self-quantising form carries at most four samples");
+        if constexpr (FQ == 1) gemv_i8_specialised<FMT, 3, 2, true>(a);
+        else gemv_i8_specialised<FMT, 2, 4, false>(a);
+        return;
+    }
     using F = I8Fmt<FMT>;
     constexpr int KL = F::KL, NMF = F::NMF, G = 4;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
@@ -472,21 +729,7 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
         }
     };
 
-    // The self-quantising variant requests the activations of its first scale chunk before the
-    // weights: loads complete in order, and the quantiser should not wait behind the weight stream.
-    constexpr int QN = FQ ? FQ : 1;
-    QuantRegs<FMT, QN> qr;
-    const uint32_t spc = ((uint32_t)nb + QN - 1) / QN;         // sample groups per chunk
-    const uint32_t nch_first = chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks;
-    auto unit_load = [&](uint32_t ch0, uint32_t ui) {
-        const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
-        const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
-        quant_load<FMT, QN>(qr, a.x + (size_t)sbase * K, K, (ch0 + chl) * a.kc, a.kc, ns, lane);
-    };
-    if constexpr (FQ != 0) {
-        if ((uint32_t)wave < nch_first * spc) unit_load(0u, (uint32_t)wave);
-    }
-    // then the first weight group (PD groups in flight; two measured slower than one)
+    // the first weight group
     constexpr int PD = 1;
     uint4 nxt[PD][G];
 #pragma unroll
@@ -495,38 +738,19 @@ __global__ __launch_bounds__(FQ ? 512 : MT <= 4 ? 1024 : 256) void sp_gemv_i8mfm
         for (int u = 0; u < G; ++u) nxt[d][u] = load_blk((uint32_t)(d * G + u));
 
     // scale records of all chunks
-    if constexpr (!FQ) {
-        for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
-            const int *d = a.dsum + (size_t)i * 4;
-            meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
-        }
+    for (uint32_t i = t; i < a.nchunks * (uint32_t)nb; i += nthreads) {
+        const int *d = a.dsum + (size_t)i * 4;
+        meta[i] = make_int4(__float_as_int(a.inv[i]), d[0], d[1], d[2]);
     }
 
     uint32_t q = 0;                                            // this wave's block counter
     for (uint32_t ch0 = 0; ch0 < a.nchunks; ch0 += chunks_per_stage) {
         const uint32_t nch = ch0 + chunks_per_stage <= a.nchunks ? chunks_per_stage : a.nchunks - ch0;
         if (ch0) __syncthreads();                             // previous stage fully consumed
-        if constexpr (!FQ) {
+        {
             const uint4 *src = reinterpret_cast<const uint4 *>(a.aq + (size_t)ch0 * kcb * blk_bytes);
             const uint32_t pieces = nch * kcb * (blk_bytes / 16u);
             for (uint32_t i = t; i < pieces; i += nthreads) reinterpret_cast<uint4 *>(A_lds)[i] = src[i];
-        } else {
-            // every wave takes whole scale chunks of this stage, FQ samples at once
-            for (uint32_t ui = (uint32_t)wave; ui < nch * spc; ui += nthreads / 64u) {
-                if (ch0 != 0 || ui != (uint32_t)wave) unit_load(ch0, ui);      // the first one is on its way
-                const uint32_t chl = ui / spc, sbase = (ui % spc) * QN;
-                const int ns = nb - (int)sbase < QN ? nb - (int)sbase : QN;
-                quant_finish<FMT, QN>(qr, a.kc, ns, lane,
-                    [&](uint32_t s, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
-                        uint8_t *dst = A_lds + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + sbase + s) * 48 + w * 4;
-                        *reinterpret_cast<uint32_t *>(dst) = d0;
-                        *reinterpret_cast<uint32_t *>(dst + 16) = d1;
-                        *reinterpret_cast<uint32_t *>(dst + 32) = d2;
-                    },
-                    [&](uint32_t s, int4 md) {
-                        if (lane == 0) meta[(size_t)(ch0 + chl) * nb + sbase + s] = md;
-                    });
-            }
         }
         __syncthreads();
         const uint8_t *rec = A_lds + (size_t)ks_id * blk_bytes;
