@@ -669,7 +669,11 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
     const uint32_t max_waves = MT > 4 ? 4u : 16u;             // register budget of the wide tiles
     // up to four samples: the GEMV workgroups quantise the activations themselves
     const bool fused = MT == 1;
-    const uint32_t ks_cap = 2048u / (4u * KL);                 // a scale chunk is a whole number of fetch groups
+    // self-quantising form: K shares of whole 128-byte lines in fetch groups of two blocks up to 64 MiB of weights,
+    // of single blocks in groups of four beyond (gemv_i8_specialised has the measurements)
+    const bool line_shares = fused && (uint64_t)L.N * L.K * I8Fmt<FMT>::bits / 8u <= (64ull << 20);
+    const uint32_t G = line_shares ? 2u : 4u;                  // blocks per fetch group
+    const uint32_t ks_cap = 2048u / (G * KL);                  // a scale chunk is a whole number of fetch groups
                                                                // and at most 2048 codes (one wave's batch of loads)
     uint32_t rw, ks;
     if (fused) {
@@ -689,9 +693,9 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
         ks = max_waves / rw > 8u ? 8u : max_waves / rw;
         if (ks > ks_cap) ks = ks_cap;
     }
-    // one fetch group (4 blocks of every K share) must fit the row, the stage budget and one scale chunk
-    while (ks > 1 && (kblocks < 4u * ks || 4u * ks * blk_bytes > budget)) ks >>= 1;
-    const uint32_t group_blocks = 4u * ks;
+    // one fetch group (G blocks of every K share) must fit the row, the stage budget and one scale chunk
+    while (ks > 1 && (kblocks < G * ks || G * ks * blk_bytes > budget)) ks >>= 1;
+    const uint32_t group_blocks = G * ks;
     // scale chunk: about 2048 codes, a whole number of fetch groups, and small enough for one LDS stage
     uint32_t kc_blocks = 2048u / KL;
     if (kc_blocks > budget / blk_bytes) kc_blocks = budget / blk_bytes;
@@ -721,12 +725,13 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
         a.stage_blocks = stage;
         if (lds < red_bytes) lds = red_bytes;
         lds += a.meta_bytes;
-        // one quant wave per (scale chunk, sample) of the first stage, at most eight
+        // one quant wave per (scale chunk, sample) of the first stage, at most eight.  (Cutting a chunk into slices so
+        // that eight waves quantise a K of fewer chunks, the slices' maxima meeting in LDS, was measured: 0.7-0.9 us
+        // slower per layer on 8192-wide INT2 / INT8 layers.)
         const uint32_t units = (stage / kc_blocks < a.nchunks ? stage / kc_blocks : a.nchunks) * n;
         a.qw = units < 8u ? units : 8u;
-        // how a K share's blocks are chosen: see gemv_i8_specialised
-        if ((uint64_t)L.N * L.K * I8Fmt<FMT>::bits / 8u > (64ull << 20)) launch_gemv_i8_mt<FMT, 1, 2>(a, grid, (waves + a.qw) * 64, lds);
-        else launch_gemv_i8_mt<FMT, 1, 1>(a, grid, (waves + a.qw) * 64, lds);
+        if (line_shares) launch_gemv_i8_mt<FMT, 1, 1>(a, grid, (waves + a.qw) * 64, lds);
+        else launch_gemv_i8_mt<FMT, 1, 2>(a, grid, (waves + a.qw) * 64, lds);
         return true;
     }
     // LDS stage: everything if it fits the budget, else whole scale chunks

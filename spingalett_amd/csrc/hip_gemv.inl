@@ -241,99 +241,95 @@ __device__ __forceinline__ void quant_word(const float4 (&v)[I8Fmt<FMT>::WK / 4]
     }
 }
 
-// One wave quantises one scale chunk (kc <= 2048 codes starting at code kbase) of up to NS
-// samples (rows xr, xr + K, ...; ns of them are real): every lane fetches its words'
-// activations in one batch of loads (quant_load), the wave agrees on the largest magnitude per
-// sample, and each lane converts what it holds (quant_finish).
+// One wave quantises up to 2048 consecutive activations of one sample (a scale chunk, or a slice of one: `len` codes
+// starting at code kbase of row xr): every lane fetches its words' activations in one batch of loads (quant_load),
+// the wave finds the largest magnitude (quant_amax), and each lane converts what it holds with the scale that the
+// chunk's largest magnitude gives (quant_digits).
 // A 64-byte weight segment (block) is spread over 4 lane groups g of 16 bytes = 4 words w;
 // word w holds WK codes; after unpacking, MFMA u of that block takes byte i of word w from code
 //   INT8: 4w+i (u = 0)      INT4: 8w + 2i + u      INT2: 16w + 4i + u
-// of the lane group.  store(sample, block in chunk, u, g, w, d0, d1, d2) receives the operand
-// words; done(sample, {bits of 2^-p, sum d0, sum d1, sum d2}) the scale record (same in every lane).
-template <int FMT, int NS>
+// of the lane group.  store(block, u, g, w, d0, d1, d2) receives the operand words (block counted from kbase);
+// the result is the scale record {bits of 2^-p, sum d0, sum d1, sum d2} of what this wave converted (same in every lane).
+template <int FMT>
 struct QuantRegs {
     static constexpr int MAXIT = 2048 / (64 * I8Fmt<FMT>::WK);
     static constexpr int F4 = I8Fmt<FMT>::WK / 4;
-    float4 v[NS][MAXIT][F4];
+    float4 v[MAXIT][F4];
 };
 
-template <int FMT, int NS>
-__device__ __forceinline__ void quant_load(QuantRegs<FMT, NS> &q, const float *xr, uint32_t K, uint32_t kbase,
-                                           uint32_t kc, int ns, int lane)
+template <int FMT>
+__device__ __forceinline__ void quant_load(QuantRegs<FMT> &q, const float *xr, uint32_t K, uint32_t kbase, uint32_t len, int lane)
 {
     using F = I8Fmt<FMT>;
-    constexpr int KL = F::KL, WK = F::WK, F4 = WK / 4, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr int KL = F::KL, WK = F::WK, F4 = WK / 4, MAXIT = QuantRegs<FMT>::MAXIT;
     constexpr uint32_t WPB = KL / WK;                            // words per block (16)
-    const uint32_t iters = kc / (64u * WK);
+    const uint32_t iters = len / (64u * WK);
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        const float *xs = xr + (size_t)(s < ns ? s : 0) * K;
+    for (int it = 0; it < MAXIT; ++it) {
+        const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+        const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+        const uint32_t kw = kbase + blk * KL + gg * (KL / 4) + w * WK;     // first code of the word
+        const bool valid = (uint32_t)it < iters && kw < K;                  // rows are whole numbers of words
+        const float4 *src = reinterpret_cast<const float4 *>(xr + (valid ? kw : 0u));
 #pragma unroll
-        for (int it = 0; it < MAXIT; ++it) {
-            const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
-            const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
-            const uint32_t kw = kbase + blk * KL + gg * (KL / 4) + w * WK;     // first code of the word
-            const bool valid = (uint32_t)it < iters && kw < K;                  // rows are whole numbers of words
-            const float4 *src = reinterpret_cast<const float4 *>(xs + (valid ? kw : 0u));
-#pragma unroll
-            for (int c = 0; c < F4; ++c) {
-                float4 t = src[c];
-                if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                q.v[s][it][c] = t;
-            }
+        for (int c = 0; c < F4; ++c) {
+            float4 t = src[c];
+            if (!valid) t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            q.v[it][c] = t;
         }
     }
 }
 
-template <int FMT, int NS, class Store, class Done>
-__device__ __forceinline__ void quant_finish(const QuantRegs<FMT, NS> &q, uint32_t kc, int ns, int lane, Store store, Done done)
+// largest |x| the wave holds, as its bit pattern: orders like the value, and infinities and NaNs sort last
+template <int FMT>
+__device__ __forceinline__ uint32_t quant_amax(const QuantRegs<FMT> &q)
+{
+    uint32_t lm = 0u;
+#pragma unroll
+    for (int it = 0; it < QuantRegs<FMT>::MAXIT; ++it)
+#pragma unroll
+        for (int c = 0; c < QuantRegs<FMT>::F4; ++c) {
+            const float4 t = q.v[it][c];
+            const uint32_t mx = max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu);
+            const uint32_t mz = max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu);
+            lm = max(lm, max(mx, mz));
+        }
+    return wave_max_u(lm);
+}
+
+template <int FMT, class Store>
+__device__ __forceinline__ int4 quant_digits(const QuantRegs<FMT> &q, uint32_t amax, uint32_t len, int lane, Store store)
 {
     using F = I8Fmt<FMT>;
-    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, MAXIT = QuantRegs<FMT, NS>::MAXIT;
+    constexpr int KL = F::KL, NMF = F::NMF, WK = F::WK, MAXIT = QuantRegs<FMT>::MAXIT;
     constexpr uint32_t WPB = KL / WK;
-    const uint32_t iters = kc / (64u * WK);
+    const uint32_t iters = len / (64u * WK);
+    int e = (int)(amax >> 23) - 127;
+    if (e < -126) e = -126;
+    int p = 21 - e;                                              // |X| < 2^22: the top digit stays inside INT8
+    p = p > 126 ? 126 : p;
+    // A chunk that holds an infinity or a NaN cannot be written in digits: its record carries a NaN instead of
+    // 2^-p, which turns the sample's sums into NaN, and the epilogue redoes those outputs in FP32 arithmetic so
+    // that infinities and NaNs come out as cblas_sgemv / the FP32 dot product give them (Network.c:229-245).
+    const bool finite = amax < 0x7F800000u;
+    const bool live = amax != 0u && finite;                      // an all-zero chunk contributes nothing
+    const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
+    int ds0 = 0, ds1 = 0, ds2 = 0;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        if (s >= ns) break;
-        // largest |x| of the chunk as its bit pattern: orders like the value, and infinities and NaNs sort last
-        uint32_t lm = 0u;
+    for (int it = 0; it < MAXIT; ++it) {
+        if ((uint32_t)it < iters) {
+            const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
+            const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
+            uint32_t d0[NMF], d1[NMF], d2[NMF];
+            quant_word<FMT>(q.v[it], scale, d0, d1, d2, ds0, ds1, ds2);
 #pragma unroll
-        for (int it = 0; it < MAXIT; ++it)
-#pragma unroll
-            for (int c = 0; c < F::WK / 4; ++c) {
-                const float4 t = q.v[s][it][c];
-                const uint32_t mx = max(__float_as_uint(t.x) & 0x7FFFFFFFu, __float_as_uint(t.y) & 0x7FFFFFFFu);
-                const uint32_t mz = max(__float_as_uint(t.z) & 0x7FFFFFFFu, __float_as_uint(t.w) & 0x7FFFFFFFu);
-                lm = max(lm, max(mx, mz));
-            }
-        const uint32_t amax = wave_max_u(lm);
-        int e = (int)(amax >> 23) - 127;
-        if (e < -126) e = -126;
-        int p = 21 - e;                                          // |X| < 2^22: the top digit stays inside INT8
-        p = p > 126 ? 126 : p;
-        // A chunk that holds an infinity or a NaN cannot be written in digits: its record carries a NaN instead of
-        // 2^-p, which turns the sample's sums into NaN, and the epilogue redoes those outputs in FP32 arithmetic so
-        // that infinities and NaNs come out as cblas_sgemv / the FP32 dot product give them (Network.c:229-245).
-        const bool finite = amax < 0x7F800000u;
-        const bool live = amax != 0u && finite;                  // an all-zero chunk contributes nothing
-        const float scale = live ? __uint_as_float((uint32_t)(p + 127) << 23) : 0.0f;
-        int ds0 = 0, ds1 = 0, ds2 = 0;
-#pragma unroll
-        for (int it = 0; it < MAXIT; ++it) {
-            if ((uint32_t)it < iters) {
-                const uint32_t wl = (uint32_t)it * 64u + (uint32_t)lane;
-                const uint32_t blk = wl / WPB, r = wl % WPB, gg = r >> 2, w = r & 3u;
-                uint32_t d0[NMF], d1[NMF], d2[NMF];
-                quant_word<FMT>(q.v[s][it], scale, d0, d1, d2, ds0, ds1, ds2);
-#pragma unroll
-                for (int u = 0; u < NMF; ++u) store((uint32_t)s, blk, (uint32_t)u, gg, w, d0[u], d1[u], d2[u]);
-            }
+            for (int u = 0; u < NMF; ++u) store(blk, (uint32_t)u, gg, w, d0[u], d1[u], d2[u]);
         }
-        ds0 = wave_sum_i(ds0);
-        ds1 = wave_sum_i(ds1);
-        ds2 = wave_sum_i(ds2);
-        done((uint32_t)s, make_int4(live ? (int)((uint32_t)(127 - p) << 23) : finite ? 0 : 0x7FC00000, ds0, ds1, ds2));
     }
+    ds0 = wave_sum_i(ds0);
+    ds1 = wave_sum_i(ds1);
+    ds2 = wave_sum_i(ds2);
+    return make_int4(live ? (int)((uint32_t)(127 - p) << 23) : finite ? 0 : 0x7FC00000, ds0, ds1, ds2);
 }
 
 // Quantise kernel (n > 4): one wave per sample and scale chunk, four to a workgroup.
@@ -350,22 +346,20 @@ __global__ __launch_bounds__(256) void sp_quant_x(const GemvI8Args a)
     if (rec >= a.nchunks * (uint32_t)a.nb) return;
     const uint32_t ch = rec / (uint32_t)a.nb, s0 = rec % (uint32_t)a.nb;
     const uint32_t nblk = a.kc / KL;                         // blocks per chunk (last chunk zero-padded)
-    QuantRegs<FMT, 1> qr;
-    quant_load<FMT, 1>(qr, a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, 1, lane);
-    quant_finish<FMT, 1>(qr, a.kc, 1, lane,
-        [&](uint32_t, uint32_t blk, uint32_t u, uint32_t g, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+    QuantRegs<FMT> qr;
+    quant_load<FMT>(qr, a.x + (size_t)s0 * a.L.K, a.L.K, ch * a.kc, a.kc, lane);
+    const int4 md = quant_digits<FMT>(qr, quant_amax<FMT>(qr), a.kc, lane,
+        [&](uint32_t blk, uint32_t u, uint32_t g, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
             uint8_t *dst = a.aq + (((((size_t)ch * nblk + blk) * NMF + u) * 4 + g) * (size_t)a.nb + s0) * 48 + w * 4;
             *reinterpret_cast<uint32_t *>(dst) = d0;
             *reinterpret_cast<uint32_t *>(dst + 16) = d1;
             *reinterpret_cast<uint32_t *>(dst + 32) = d2;
-        },
-        [&](uint32_t, int4 md) {
-            if (lane == 0) {
-                a.inv[rec] = __int_as_float(md.x);
-                int *d = a.dsum + (size_t)rec * 4;
-                d[0] = md.y; d[1] = md.z; d[2] = md.w; d[3] = 0;
-            }
         });
+    if (lane == 0) {
+        a.inv[rec] = __int_as_float(md.x);
+        int *d = a.dsum + (size_t)rec * 4;
+        d[0] = md.y; d[1] = md.z; d[2] = md.w; d[3] = 0;
+    }
 }
 
 // Self-quantising form for up to four samples: one launch per layer, the waves of a workgroup specialised.
@@ -421,37 +415,34 @@ __device__ __forceinline__ void gemv_i8_specialised(const GemvI8Args &a)
     if (wave >= sw) {
         // ---- quant wave
         const uint32_t qid = wave - sw;
-        QuantRegs<FMT, 1> qr;
-        // The first unit's activations are requested before any weight and have arrived when the stream waves are let
-        // go (barrier "go"): the memory pipeline of a compute unit returns data in request order, and activations
-        // queued behind a few megabytes of weight requests arrive microseconds later.
-        {
-            const uint32_t nch0 = cps <= a.nchunks ? cps : a.nchunks;
-            if (qid < nch0 * nb) {
-                quant_load<FMT, 1>(qr, a.x + (size_t)(qid % nb) * K, K, (qid / nb) * a.kc, a.kc, 1, lane);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
-            __syncthreads();                                      // barrier "go"
+        QuantRegs<FMT> qr;
+        auto store_to = [&](uint8_t *buf, uint32_t blk0, uint32_t smp) {
+            return [=](uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
+                uint8_t *dst = buf + ((((size_t)(blk0 + blk) * NMF + u) * 4 + gg) * (size_t)nb + smp) * 48 + w * 4;
+                *reinterpret_cast<uint32_t *>(dst) = d0;
+                *reinterpret_cast<uint32_t *>(dst + 16) = d1;
+                *reinterpret_cast<uint32_t *>(dst + 32) = d2;
+            };
+        };
+        // The activations of a wave's first unit are requested before any weight and have arrived when the stream
+        // waves are let go (barrier "go").
+        const uint32_t nch0 = cps <= a.nchunks ? cps : a.nchunks;
+        if (qid < nch0 * nb) {
+            quant_load<FMT>(qr, a.x + (size_t)(qid % nb) * K, K, (qid / nb) * a.kc, a.kc, lane);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
+        __syncthreads();                                      // barrier "go"
         for (uint32_t s = 0; s < nstages; ++s) {
             const uint32_t ch0 = s * cps, nch = ch0 + cps <= a.nchunks ? cps : a.nchunks - ch0;
             uint8_t *buf = A_lds + (size_t)(s & 1u) * buf_bytes;
             for (uint32_t ui = qid; ui < nch * nb; ui += a.qw) {
                 const uint32_t chl = ui / nb, smp = ui % nb;
-                if (s != 0 || ui != qid)                          // the first unit is in the registers already
-                    quant_load<FMT, 1>(qr, a.x + (size_t)smp * K, K, (ch0 + chl) * a.kc, a.kc, 1, lane);
-                quant_finish<FMT, 1>(qr, a.kc, 1, lane,
-                    [&](uint32_t, uint32_t blk, uint32_t u, uint32_t gg, uint32_t w, uint32_t d0, uint32_t d1, uint32_t d2) {
-                        uint8_t *dst = buf + (((((size_t)chl * kcb + blk) * NMF + u) * 4 + gg) * (size_t)nb + smp) * 48 + w * 4;
-                        *reinterpret_cast<uint32_t *>(dst) = d0;
-                        *reinterpret_cast<uint32_t *>(dst + 16) = d1;
-                        *reinterpret_cast<uint32_t *>(dst + 32) = d2;
-                    },
-                    [&](uint32_t, int4 md) {
-                        if (lane == 0) meta[(size_t)(ch0 + chl) * nb + smp] = md;
-                    });
+                if (s != 0 || ui != qid)                      // the first unit is in the registers already
+                    quant_load<FMT>(qr, a.x + (size_t)smp * K, K, (ch0 + chl) * a.kc, a.kc, lane);
+                const int4 md = quant_digits<FMT>(qr, quant_amax<FMT>(qr), a.kc, lane, store_to(buf, chl * kcb, smp));
+                if (lane == 0) meta[(size_t)(ch0 + chl) * nb + smp] = md;
             }
-            __syncthreads();                                      // barrier s: stage s is written
+            __syncthreads();                                  // barrier s: stage s is written
         }
         if (ks > 1) {                                             // the two barriers of the K-share reduction
             __syncthreads();
