@@ -164,15 +164,23 @@ def time_workload(copies, topo, n, x_host, steps, warmup):
     return wall * 1e3 / steps, ev_ms / steps, y
 
 
-# HBM-side bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (summaries and calibration factors: profiles/sp_gemm16_big_C4_bf16_b8192.md,
-# profiles/sp_gemv_i8mfma_C3_int4_b1.md, profiles/sp_skinny16_C3_int4_b64.md).
-# Keyed by (kernel, [n, N, K]); None when not profiled.
-PROFILED_TRAFFIC = {
-    ("sp_gemm16_big", (8192, 8192, 8192)): (790488 * 2.0 + 186515 * 1.0) * 1024,
-    ("sp_gemv_i8mfma", (1, 16384, 16384)): (68204 * 2.0 + 64 * 1.0) * 1024,
-    ("sp_skinny16", (64, 16384, 16384)): ((78179 + 8215) * 2.0 + (16384 + 2048) * 1.0) * 1024,
-}
+# HBM-side bytes per launch of the dominant kernels: profiles/traffic.json, written by bench_traffic.py from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (each entry carries its counter readings, the
+# calibration factors from a plain copy of known size in the same run, and the commands).  Keyed by kernel and
+# [n, N, K]; a dominant kernel without an entry reports traffic null and a warning on stderr.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def load_traffic():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entries = json.load(f)["entries"]
+    except (OSError, ValueError, KeyError):
+        return {}
+    return {(e["kernel"], tuple(e["shape"])): e["bytes"] for e in entries}
+
+
+PROFILED_TRAFFIC = load_traffic()
 
 
 def dominant_layer(topo):
@@ -187,6 +195,9 @@ def roofline_for(copies, topo, prec, n, iters):
     K, N = topo[l - 1], topo[l]
     kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
     traffic = PROFILED_TRAFFIC.get((kernel, (n, N, K)))
+    if traffic is None:
+        print(f"bench.py: no profiled traffic for {kernel} at [n, N, K] = {[n, N, K]} in profiles/traffic.json "
+              "(bench_traffic.py adds it)", file=sys.stderr)
     if n <= 64:
         # memory regime: serialized weights + bias of the layer, FP32 inputs and outputs of the layer
         nbytes = array_payload(K * N, prec) + array_payload(N, prec) + 4 * n * (K + N)
@@ -221,7 +232,7 @@ def cpu_baseline(path, cfg, n_sample, budget_s=12.0):
                 sample=f"{n_sample} samples x {iters} iterations of the same net on host cores, {desc}")
 
 
-def run_workload(name, batches, steps, warmup, want_output=False):
+def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0.0):
     cfg = WORKLOADS[name]
     topo, prec = cfg["topo"], cfg["prec"]
     t0 = time.perf_counter()
@@ -250,6 +261,15 @@ def run_workload(name, batches, steps, warmup, want_output=False):
                 S.forward(net, x1)
             row["public_forward_us"] = (time.perf_counter() - t1) / 200 * 1e6
         rows.append(row)
+    if cpu_budget_s > 0:
+        # one CPU leg per configuration (a bounded sample of its largest batch), attached to every row of it
+        sample = min(max(batches), 64 if flops_per_sample(topo) > 1e8 else 4096)
+        try:
+            cpu = cpu_baseline(path, cfg, sample, cpu_budget_s)
+        except Exception as e:
+            cpu = dict(error=str(e))
+        for row in rows:
+            row["cpu_baseline"] = cpu
     return dict(net=net, path=path, copies=copies, clones=clones, rows=rows, build_s=build_s)
 
 
@@ -387,7 +407,7 @@ def main():
             if name == args.workload:
                 continue
             try:
-                w = run_workload(name, WORKLOADS[name]["batches"], 50, 3)
+                w = run_workload(name, WORKLOADS[name]["batches"], 50, 3, cpu_budget_s=0.0 if args.no_cpu else 2.0)
                 extra += w["rows"]
                 release(w)
             except Exception as e:  # keep the headline even if an extra configuration fails

@@ -876,6 +876,8 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
     }
     p.ct = p.NC <= 32 ? 1 : 2;
     p.cblocks = (p.NC + 32u * p.ct - 1) / (32u * p.ct);
+    // two row tiles per wave only where that still leaves 128 workgroups per K split: on smaller layers it was measured
+    // slower at every sample count (16384 x 16384 INT4 at 64 samples 90 against 57 us, 8192 x 8192 INT2 33 against 23 us)
     p.rt = (p.R + 255u) / 256u * p.cblocks >= 128u ? 2 : 1;
     p.row_blocks = (p.R + 128u * p.rt - 1) / (128u * p.rt);
     const uint32_t chunks = (K + bkc - 1) / bkc;
@@ -987,12 +989,6 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
             static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
             (void)once;
             kern<<<grid, 512, lds, g_stream>>>(g);
-        } else if (getenv("SPHIP_GEMM_VARIANT") && atoi(getenv("SPHIP_GEMM_VARIANT")) == 4) {
-            constexpr size_t lds = 2 * (256 + 256) * 64 * sizeof(uint16_t);
-            auto kern = sp_gemm16_big<FMT, F16T, 2, 2, 4, 4>;
-            static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-            (void)once;
-            kern<<<grid, 256, lds, g_stream>>>(g);
         } else {
             constexpr size_t lds = 2 * (256 + 256) * 64 * sizeof(uint16_t);
             auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 4, 2>;
