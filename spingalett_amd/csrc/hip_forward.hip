@@ -83,6 +83,22 @@ int fail_hip(const char *what, hipError_t e)
         if (e_ != hipSuccess) return fail_hip(#expr, e_);         \
     } while (0)
 
+// The two events of a timed region; destroyed on every way out of the function that holds them.
+struct TimingEvents {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int create()
+    {
+        HCHECK(hipEventCreate(&e0));
+        HCHECK(hipEventCreate(&e1));
+        return 0;
+    }
+    ~TimingEvents()
+    {
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+    }
+};
+
 hipStream_t g_stream = nullptr;
 // Routing state of the calling thread.  The launch_* functions below decide which kernel a layer takes and launch it;
 // with `dry` set they only decide (nothing is enqueued), which is how sphip_layer_kernel_name answers without side
@@ -1702,17 +1718,15 @@ static int time_common(sphip_net *const *nets, int count, const float *d_x, uint
         if (check_uploaded(nets[i])) return 1;
         if (reserve(nets[i], n, false)) return 1;
     }
-    hipEvent_t e0, e1;
-    HCHECK(hipEventCreate(&e0));
-    HCHECK(hipEventCreate(&e1));
+    TimingEvents ev;
+    if (ev.create()) return 1;
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     int rc = 0;
     HCHECK(hipEventRecord(e0, g_stream));
     for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward(nets[it % count], nets[it % count]->workspace(), d_x, n, d_y, flags, only_layer);
     hipError_t e = hipEventRecord(e1, g_stream);
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     if (rc) return rc;
     if (e != hipSuccess) return fail_hip("sphip_time", e);
     return 0;

@@ -612,17 +612,15 @@ int sphip_time_train_step(sphip_net *net, const float *d_x, const float *d_targe
 {
     if (!net || !d_x || !d_targets || n == 0 || !args || iters <= 0 || !ms) return fail_msg("sphip_time_train_step: invalid argument");
     if (sphip_train_step(net, d_x, d_targets, n, args, SPHIP_X_ON_DEVICE, nullptr)) return 1;      // sizes every buffer
-    hipEvent_t e0, e1;
-    HCHECK(hipEventCreate(&e0));
-    HCHECK(hipEventCreate(&e1));
+    TimingEvents ev;
+    if (ev.create()) return 1;
+    hipEvent_t e0 = ev.e0, e1 = ev.e1;
     int rc = 0;
     HCHECK(hipEventRecord(e0, g_stream));
     for (int it = 0; it < iters && !rc; ++it) rc = sphip_train_step(net, d_x, d_targets, n, args, SPHIP_X_ON_DEVICE, nullptr);
     hipError_t e = hipEventRecord(e1, g_stream);
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     if (rc) return rc;
     if (e != hipSuccess) return fail_hip("sphip_time_train_step", e);
     return 0;
