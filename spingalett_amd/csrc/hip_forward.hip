@@ -234,6 +234,17 @@ __device__ __forceinline__ float apply_act(float x, int act)
     }
 }
 
+// the same for the activations that need no transcendental function (a caller has dealt with the other two)
+__device__ __forceinline__ float apply_act_cheap(float x, int act)
+{
+    switch (act) {
+    case A_RELU:    return x > 0.0f ? x : 0.0f;
+    case A_LEAKY:   return x > 0.0f ? x : 0.01f * x;
+    case A_FOO52:   return x > 1.0f ? 1.0f + 0.01f * (x - 1.0f) : (x < 0.0f ? 0.01f * x : x);
+    default:        return x;
+    }
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
 {
     uint32_t u = __float_as_uint(x);
@@ -797,7 +808,7 @@ uint32_t gemm16_tile_rows(uint32_t M)
 uint32_t gemm16_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 {
     const uint32_t bm = gemm16_tile_rows(M);
-    const uint32_t tiles = ((M + bm - 1) / bm) * ((N + 255u) / 256u), ktiles = K / 64u;
+    const uint32_t tiles = ((M + bm - 1) / bm) * ((N + 255u) / 256u), ktiles = (K + 63u) / 64u;
     *kper = 0;
     if (tiles >= 192u || ktiles < 16u) return 1;
     uint32_t splits = (256u + tiles - 1) / tiles;
@@ -827,20 +838,22 @@ struct ThinPlan {
     int nw;                // waves per workgroup in that case (4 or 8)
     uint32_t R, NC;        // streamed rows, thin rows
     int rt, ct;
+    int nwv;               // waves per workgroup of sp_skinny16
     uint32_t splits, kper, row_blocks, cblocks;
 };
 
 // Largest batch the weight-streaming kernel takes before the tiled GEMM does better (which runs from 65 samples up, a
-// partly filled row of 256 x 256 tiles).  Measured on whole nets: 8192-wide BF16 layers 417 / 439 / 475 us at 72 / 96 /
-// 128 samples through the GEMM against 468 / 486 / 502 us streaming (and 576 against 918 us at 256); 16384-wide INT4
-// 281 / 305 us at 192 / 256 against 366 / 369 us, but 257 / 263 us at 96 / 128 against 213 / 233 us; 8192-wide INT2 still
-// 8 % better streaming at 256.  The fewer bytes a code has, the longer re-reading the weights per block of 64 samples pays.
+// partly filled row of 256 x 256 tiles).  Measured per layer, streaming against tiles, at 128 and 192 samples:
+// 8192 x 8192 BF16 57 / 107 against 48 / 57 us (tiles from 65 samples: 54 against 43 us there); 8192 x 8192 INT8 36 / 66
+// against 41 / 54 us and 16384 x 16384 INT8 108 / 175 against 119 / 145 us (tiles from 129); 16384 x 16384 INT4 82 / 141
+// against 104 / 143 us, 4096 x 16384 INT4 34 / 54 against 52 / 71 us, 8192 x 8192 INT2 29 / 44 against 40 / 52 us (streaming
+// up to 256).  The fewer bytes a code has, the longer re-reading the weights per block of 64 samples pays.
 // Layers of a few megabytes stay with the streaming kernel up to 256 samples (the 784-512-1000-10 INT8 net: 36 us
 // against 57 us at 256 samples).
 uint32_t thin_max_samples(int fmt, uint32_t N, uint32_t K)
 {
     if ((uint64_t)N * K * (uint64_t)fmt_bits(fmt) / 8u <= (8ull << 20)) return 256u;
-    return fmt_bits(fmt) == 16 ? 64u : fmt == I2 ? 256u : 128u;
+    return fmt_bits(fmt) == 16 ? 64u : fmt == I8 ? 128u : 256u;
 }
 
 // mode_b streams 16-bit activations (fmt = the activation type), mode a the weights
@@ -892,13 +905,20 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
     }
     p.ct = p.NC <= 32 ? 1 : 2;
     p.cblocks = (p.NC + 32u * p.ct - 1) / (32u * p.ct);
-    // two row tiles per wave only where that still leaves 128 workgroups per K split: on smaller layers it was measured
-    // slower at every sample count (16384 x 16384 INT4 at 64 samples 90 against 57 us, 8192 x 8192 INT2 33 against 23 us)
-    p.rt = (p.R + 255u) / 256u * p.cblocks >= 128u ? 2 : 1;
-    p.row_blocks = (p.R + 128u * p.rt - 1) / (128u * p.rt);
+    // Waves per workgroup, and the number of workgroups the K split aims at.  Every workgroup fetches the thin block
+    // of its K share once, so eight waves (256 streamed rows) halve that traffic; they pay from 16384 streamed rows,
+    // or from 8192 with several blocks of thin rows (16384 x 16384 INT4: 38.7 / 50.4 / 83 us at 32 / 64 / 128 samples
+    // against 42.2 / 57.0 / 124; 8192 x 8192 INT2 at 256 samples 45 against 53 us), four waves stay better on smaller
+    // layers (8192 x 8192 INT8 at 64 samples 27.3 against 29.0 us).  One workgroup per compute unit is the target:
+    // twice as many K splits write twice the partial sums (16384 x 16384 INT4 at 64 samples 67 us, 8192 x 8192 INT8
+    // 38 us), half as many leave compute units idle (74 us).  Two row tiles per wave were slower wherever tried.
+    p.rt = 1;
+    p.nwv = (p.R >= 16384u || (p.R >= 8192u && p.cblocks > 1u)) ? 8 : 4;
+    const uint32_t target = 256u;
+    p.row_blocks = (p.R + 32u * p.nwv * p.rt - 1) / (32u * p.nwv * p.rt);
     const uint32_t chunks = (K + bkc - 1) / bkc;
     const uint32_t wgs = p.row_blocks * p.cblocks;
-    uint32_t splits = (512u + wgs - 1) / wgs;
+    uint32_t splits = (target + wgs - 1) / wgs;
     if (splits > 16u) splits = 16u;
     if (splits > chunks / 2u) splits = chunks / 2u;
     if (splits < 1u) splits = 1u;
@@ -908,16 +928,16 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
     return p;
 }
 
-template <int SFMT, bool F16T, int RT, int CT>
+template <int SFMT, bool F16T, int RT, int CT, int NWV = 4>
 void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
 {
     if (tl_route.dry) return;
     constexpr size_t lds = 2 * 32 * CT * SkinnyFmt<SFMT>::PITCH;
-    auto kern = sp_skinny16<SFMT, F16T, RT, CT>;
+    auto kern = sp_skinny16<SFMT, F16T, RT, CT, NWV>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
     (void)once;
     const uint32_t gx = p.cblocks > 1 ? (p.row_blocks + 7u) / 8u * 8u * p.cblocks : p.row_blocks;
-    kern<<<dim3(gx, p.splits, 1), 256, lds, g_stream>>>(a);
+    kern<<<dim3(gx, p.splits, 1), 64 * NWV, lds, g_stream>>>(a);
 }
 
 template <int SFMT, bool F16T, int NCP, int NW>
@@ -949,14 +969,18 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
         } else {
             launch_thin_kw<SFMT, F16T, 8, 4>(a, p);
         }
-    } else if (p.rt == 2) {
-        if (p.ct == 2) launch_thin_inst<SFMT, F16T, 2, 2>(a, p); else launch_thin_inst<SFMT, F16T, 2, 1>(a, p);
+    } else if (p.nwv == 8) {
+        if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2, 8>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1, 8>(a, p);
     } else {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1>(a, p);
     }
     if (p.splits > 1 && !tl_route.dry) {
         const uint64_t total = (uint64_t)a.NC * a.R;
-        sp_skinny_reduce<F16T><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(a, p.splits);
+        // four rows per thread where they are neighbours in the workspace and in C, and both are 16-byte aligned
+        const bool vec = !a.mode_b && a.R % 4u == 0 && (reinterpret_cast<uintptr_t>(a.ws) & 15u) == 0 &&
+                         (reinterpret_cast<uintptr_t>(a.C) & 15u) == 0;
+        if (vec) sp_skinny_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(a, p.splits);
+        else sp_skinny_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(a, p.splits);
     }
 }
 
@@ -992,7 +1016,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const uint32_t big_tiles = ((M + bm - 1) / bm) * ((L.N + 255u) / 256u);
     const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
-    if (aligned && L.K % 64u == 0 && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
+    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
         else g.ws = ctx.ws;
         const dim3 grid(big_tiles, g.ws ? splits : 1u);

@@ -320,6 +320,12 @@ __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
 // does not track these loads: the caller waits with s_waitcnt vmcnt before the data is read.
 __device__ __forceinline__ void lds_dma16(uint32_t lds_addr, uint32_t voff, const void *sbase)
 {
+    // Both are uniform by construction; saying so keeps them in scalar registers where the compiler's own analysis
+    // gives up (it folds the intrinsic away where it does not).
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
+    const uint64_t b = reinterpret_cast<uint64_t>(sbase);
+    sbase = reinterpret_cast<const void *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 
@@ -340,8 +346,11 @@ __device__ __forceinline__ void frag_reads(u32x4 *dst, uint32_t addr)
 }
 
 // ---------------------------------------------------------------------------
-// Large-tile variant of the 16-bit MFMA GEMM (K a multiple of 64, rows 16-byte
-// aligned).  WM x WN waves, each TM x TN tiles of 32x32; BK = 64.
+// Large-tile variant of the 16-bit MFMA GEMM (rows 16-byte aligned).  WM x WN waves,
+// each TM x TN tiles of 32x32; BK = 64.  A K that is not a multiple of 64 leaves a
+// partial K tile, which is processed first: its lanes past the end of a row fetch the
+// row's element k0 instead (always inside the array) and overwrite what they fetched
+// with zeros once it has landed.
 //   * LDS rows hold 64 elements = eight 16-byte chunks, unpadded; chunk c of row
 //     r sits at position c ^ ((r >> 1) & 7).  A 128-bit fragment read is served 16
 //     lanes (16 consecutive rows, 256 bytes = all 64 banks) per cycle: rows of equal
@@ -433,6 +442,10 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
         }
     }
+    // which 8 elements of a 64-element tile row this lane fetches: the same for every load it issues, because
+    // the rows of two of its loads are a multiple of 16 apart
+    static_assert(NWAVES % 2 == 0 && HALF % 2 == 0, "the swizzle of a lane's loads must not depend on the load");
+    const uint32_t kchunk = (uint32_t)((lane & 7) ^ ((((wave & (HALF - 1)) * 8 + (lane >> 3)) >> 1) & 7)) << 3;
     const char *a_base = reinterpret_cast<const char *>(g.A);
     const char *w_base = reinterpret_cast<const char *>(g.L.w);
     const size_t w_row_bytes = (size_t)K * bits / 8u;
@@ -472,6 +485,49 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
                 if (row < BN)
                     rw[i] = *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)(k0 + kc * EPL) * bits / 8u);
             }
+        }
+    };
+    // The partial K tile at k0 (prologue only).  Rows are whole 16-byte units, so a 16-byte piece lies entirely
+    // inside a row or entirely past its end; code 0 decodes to 0.
+    auto load_w_regs_tail = [&](uint32_t k0) {
+        if constexpr (!W_DIRECT) {
+            constexpr int LPR = BK / EPL;
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i) {
+                const int c = t + NT * i, row = c / LPR, kc = c % LPR;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                if (row >= BN) continue;
+                if (k0 + kc * EPL < K)
+                    rw[i] = *reinterpret_cast<const uint4 *>(g.L.w + (size_t)n * w_row_bytes + (size_t)(k0 + kc * EPL) * bits / 8u);
+                else
+                    rw[i] = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    };
+    auto issue_tail = [&](uint32_t k0) {                       // into stage 0
+        if (!loader) return;
+        const uint32_t back = k0 + kchunk < K ? 0u : kchunk * 2u;
+#pragma unroll
+        for (int d = 0; d < A_DUTY; ++d)
+            lds_dma16(lds_a + (uint32_t)(((d / PER) * NWAVES + (d % PER) * HALF) * 1024), a_voff[d] - back, a_base + (size_t)k0 * 2u);
+        if constexpr (W_DIRECT) {
+#pragma unroll
+            for (int d = 0; d < W_DUTY; ++d)
+                lds_dma16(lds_w + (uint32_t)(((d / PER) * NWAVES + (d % PER) * HALF) * 1024), w_voff[d] - back, w_base + (size_t)k0 * 2u);
+        }
+    };
+    auto zero_tail = [&](uint32_t k0) {                        // after the loads of issue_tail have landed
+        if (!loader || k0 + kchunk < K) return;
+        const uint32_t mine = (uint32_t)(wave & (HALF - 1)) * 1024u + (uint32_t)lane * 16u;
+#pragma unroll
+        for (int d = 0; d < A_DUTY; ++d)
+            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(As) + mine + ((d / PER) * NWAVES + (d % PER) * HALF) * 1024) =
+                make_uint4(0u, 0u, 0u, 0u);
+        if constexpr (W_DIRECT) {
+#pragma unroll
+            for (int d = 0; d < W_DUTY; ++d)
+                *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(Ws) + mine + ((d / PER) * NWAVES + (d % PER) * HALF) * 1024) =
+                    make_uint4(0u, 0u, 0u, 0u);
         }
     };
     auto store_w_regs = [&](int buf) {
@@ -567,15 +623,27 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     // grid y splits K for problems with too few tiles to fill the chip
     const uint32_t kbeg = g.kper ? blockIdx.y * g.kper : 0u;
     const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
-    const uint32_t ktiles = (kend - kbeg) / BK;
-    issue_direct(0, kbeg);
-    load_w_regs(kbeg);
-    store_w_regs(0);
-    asm volatile("s_waitcnt vmcnt(0)");
+    const uint32_t ktiles = (kend - kbeg + BK - 1) / BK;
+    const uint32_t tail = (kend - kbeg) % BK;              // only the last K split can have one
+    // tile 0 is the partial tile if there is one; tile s >= 1 then starts at kbeg + (s - 1) * BK
+    const uint32_t kshift = tail ? (uint32_t)BK : 0u;
+    if (tail) {
+        const uint32_t kt0 = kend - tail;
+        issue_tail(kt0);
+        load_w_regs_tail(kt0);
+        store_w_regs(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        zero_tail(kt0);
+    } else {
+        issue_direct(0, kbeg);
+        load_w_regs(kbeg);
+        store_w_regs(0);
+        asm volatile("s_waitcnt vmcnt(0)");
+    }
     __syncthreads();
     for (uint32_t kt = 0; kt < ktiles; kt += 2) {
-        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, kbeg + (kt + 1) * BK);
-        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, kbeg + (kt + 2) * BK);
+        stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, kbeg + (kt + 1) * BK - kshift);
+        if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, kbeg + (kt + 2) * BK - kshift);
     }
     if (g.ws) {
 #pragma unroll
@@ -593,6 +661,64 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
         return;
     }
     const float wscale = g.L.wscale;
+    // Output rows that are whole 16-byte units: a wave turns its 32 x (32 TN) block of each row tile around in LDS
+    // (the stages are free after the loop's last barrier; every wave has a region of its own, so no barrier is
+    // needed) and writes whole rows of the block, 16 bytes per lane, instead of one element per lane.
+    const uint32_t esz = g.out_f32 ? 4u : 2u;
+    if (((size_t)N * esz) % 16u == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0) {
+        constexpr int BW = 32 * TN;                                  // columns of a wave's block
+        float bias[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
+            bias[j] = col < N ? elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale : 0.0f;
+        }
+        // Sigmoid and tanh are kept out of the common path: a run-time switch over all activations inside the
+        // unrolled loops puts a copy of their code behind each of a lane's 16 TM TN outputs, and fetching that code
+        // took longer than the stores (a tenth of an 8192-cubed launch).  The lambda is forced inline: called, it
+        // would take the accumulators through memory.
+        auto turn = [&](auto es_c, auto slow_c) __attribute__((always_inline)) {
+            constexpr int ES = decltype(es_c)::value;
+            constexpr bool SLOW = decltype(slow_c)::value;
+            constexpr int PITCH = BW * ES + 16;                      // lanes 0-31 and 32-63 (four rows apart) on different banks
+            constexpr int LPR = BW * ES / 16;                        // lanes that write one row
+            constexpr int RPP = 64 / LPR;                            // rows per store instruction
+            char *mine = reinterpret_cast<char *>(smem) + wave * (32 * PITCH);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int rl = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                        const float pre = fmaf(acc[i][j][r], wscale, bias[j]);
+                        const float v = SLOW ? apply_act(pre, g.L.act) : apply_act_cheap(pre, g.L.act);
+                        char *dst = mine + rl * PITCH + (j * 32 + (lane & 31)) * ES;
+                        if constexpr (ES == 4) *reinterpret_cast<float *>(dst) = v;
+                        else *reinterpret_cast<uint16_t *>(dst) = f32_to_t16<F16T>(v);
+                    }
+#pragma unroll
+                for (int p = 0; p < 32 / RPP; ++p) {
+                    const int rl = p * RPP + lane / LPR, seg = lane % LPR;
+                    const uint4 v = *reinterpret_cast<const uint4 *>(mine + rl * PITCH + seg * 16);
+                    const uint32_t row = m0 + (wm * TM + i) * 32 + rl;
+                    const uint32_t col = n0 + wn * BW + seg * (16 / ES);
+                    if (row < M && col < N)                          // N is a multiple of 16 / ES: a unit is all in or all out
+                        __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w},
+                                                    reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(g.C) + ((size_t)row * N + col) * ES));
+                }
+            }
+        };
+        const bool slow = g.L.act == A_SIGMOID || g.L.act == A_TANH;
+        if (g.out_f32) {
+            if (slow) turn(std::integral_constant<int, 4>{}, std::true_type{});
+            else turn(std::integral_constant<int, 4>{}, std::false_type{});
+        } else {
+            if (slow) turn(std::integral_constant<int, 2>{}, std::true_type{});
+            else turn(std::integral_constant<int, 2>{}, std::false_type{});
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);

@@ -8,7 +8,7 @@
 // Few samples (5 .. 256) or few outputs (<= 64): one operand is a tall matrix that is
 // read exactly once (the weights, or the 16-bit activations when the layer has few
 // outputs), the other a thin 16-bit matrix of at most 64 rows per workgroup.  The tall
-// operand never touches LDS: a wave owns RT tiles of 32 streamed rows and loads them
+// operand never touches LDS: a workgroup has NWV waves (4 or 8), a wave owns RT tiles of 32 streamed rows and loads them
 // straight into registers, 16 bytes per lane, one chunk ahead; lanes 0-31 and 32-63 take
 // adjacent 16-byte pieces of a row.  The integer codes become FP16 pairs with the
 // 0x6400 | code trick (1024 + code, minus the constant, exact), which delivers the codes
@@ -140,13 +140,14 @@ __device__ __forceinline__ void load16_async(u32x4 &dst, uint32_t voff, const vo
     asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
 }
 
-template <int FMT, bool F16T, int RT, int CT>
-__global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
+template <int FMT, bool F16T, int RT, int CT, int NWV>
+__global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
 {
     using F = SkinnyFmt<FMT>;
     constexpr int EPL = F::EPL, LPC = F::LPC, BKC = F::BKC, STEPS = F::STEPS, PITCH = F::PITCH;
     constexpr int UNITS = 32 * CT * (BKC / 16);            // 16-code units of a thin chunk
-    constexpr int UPT = (UNITS + 255) / 256;
+    constexpr int NT = 64 * NWV;                           // threads of a workgroup
+    constexpr int UPT = (UNITS + NT - 1) / NT;
     constexpr int STAGE = 32 * CT * PITCH;
     extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
 
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
         cblk = rem >> 3;
         if (rblk >= a.row_blocks) return;                 // padding of the last group
     }
-    const uint32_t row0 = (rblk * 4u + (uint32_t)wave) * (32u * RT);
+    const uint32_t row0 = (rblk * (uint32_t)NWV + (uint32_t)wave) * (32u * RT);
     const uint32_t cbase = cblk * (32u * CT);
     const uint32_t kbeg = blockIdx.y * a.kper;
     const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
     bool trow_ok[UPT];
 #pragma unroll
     for (int q = 0; q < UPT; ++q) {
-        const uint32_t u = (uint32_t)t + 256u * q;
+        const uint32_t u = (uint32_t)t + (uint32_t)NT * q;
         const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
         const uint32_t c = cbase + row;
         trow_ok[q] = u < (uint32_t)UNITS && c < a.NC;
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
             const uint32_t kc0 = kbeg + last_chunk * BKC;
 #pragma unroll
             for (int q = 0; q < UPT; ++q) {
-                const uint32_t uc = ((uint32_t)t + 256u * q) % (BKC / 16);
+                const uint32_t uc = ((uint32_t)t + (uint32_t)NT * q) % (BKC / 16);
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     const bool valid = trow_ok[q] && kc0 + uc * 16u + 8u * e + 8u <= kend;
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(256) void sp_skinny16(const SkinnyArgs a)
         const uint32_t kc0 = kbeg + (ch < last_chunk ? ch : last_chunk) * BKC;
 #pragma unroll
         for (int q = 0; q < UPT; ++q) {
-            const uint32_t u = (uint32_t)t + 256u * q;
+            const uint32_t u = (uint32_t)t + (uint32_t)NT * q;
             if (u >= (uint32_t)UNITS) continue;
             const uint32_t row = u / (BKC / 16), uc = u % (BKC / 16);
             const uint32_t k = kc0 + uc * 16u;
@@ -598,16 +599,43 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     }
 }
 
-// adds the K splits of sp_skinny16 and applies bias and activation
-template <bool F16T>
+// adds the K splits of sp_skinny16 and applies bias and activation; a thread takes four neighbouring streamed rows
+// (VEC: R is a multiple of four and the rows are outputs, so they are neighbours in C as well) or one
+template <bool F16T, bool VEC>
 __global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint32_t splits)
 {
-    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
     const uint64_t total = (uint64_t)a.NC * a.R;
-    if (idx >= total) return;
-    float sum = 0.0f;
-    for (uint32_t sp = 0; sp < splits; ++sp) sum += a.ws[(uint64_t)sp * total + idx];
-    skinny_emit<F16T>(a, (uint32_t)(idx / a.R), (uint32_t)(idx % a.R), sum);
+    if constexpr (VEC) {
+        const uint64_t idx = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+        if (idx >= total) return;
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (uint32_t sp = 0; sp < splits; ++sp) {
+            const float4 v = *reinterpret_cast<const float4 *>(a.ws + (uint64_t)sp * total + idx);
+            sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+        }
+        const uint32_t c = (uint32_t)(idx / a.R), r = (uint32_t)(idx % a.R);
+        const float in[4] = {sum.x, sum.y, sum.z, sum.w};
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, r + i) * a.L.bscale;
+            v[i] = apply_act(fmaf(in[i], a.L.wscale, bias), a.L.act);
+        }
+        const size_t o = (size_t)c * a.L.N + r;
+        if (a.out_f32) {
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.C) + o) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            const uint32_t lo = (uint32_t)f32_to_t16<F16T>(v[0]) | ((uint32_t)f32_to_t16<F16T>(v[1]) << 16);
+            const uint32_t hi = (uint32_t)f32_to_t16<F16T>(v[2]) | ((uint32_t)f32_to_t16<F16T>(v[3]) << 16);
+            *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.C) + o) = make_uint2(lo, hi);
+        }
+    } else {
+        const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+        if (idx >= total) return;
+        float sum = 0.0f;
+        for (uint32_t sp = 0; sp < splits; ++sp) sum += a.ws[(uint64_t)sp * total + idx];
+        skinny_emit<F16T>(a, (uint32_t)(idx / a.R), (uint32_t)(idx % a.R), sum);
+    }
 }
 
 // unscaled integer codes of a small weight array as FP16 (the thin operand of a layer with few outputs)

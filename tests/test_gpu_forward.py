@@ -367,6 +367,10 @@ def _decoded_layer(S, fmt, N, K, seed):
     ("bf16", 12300, 584, 8), ("f16", 640, 8200, 5), ("bf16", 96, 64, 5), ("i8", 8, 4096, 1000), ("i2", 3, 2048, 4096),
     ("i4", 300, 4352, 13), ("i8", 12288, 1152, 16), ("f16", 640, 8200, 12),
     ("i8", 1, 64, 100), ("f16", 2, 8, 9), ("i2", 4, 16, 5),             # one to four outputs, K below one chunk
+    # eight-wave workgroups of the streaming kernel: from 16384 outputs, or from 8192 with more than 64 samples;
+    # ragged last row block, output counts that are and are not multiples of four (vector / scalar split-K reduction)
+    ("i4", 16384, 2048, 40), ("i2", 8192, 1024, 200), ("i4", 16500, 1056, 64), ("i8", 16390, 640, 33),
+    ("f16", 16384, 512, 9), ("i2", 20000, 768, 130),
     # few outputs, activations streamed
     ("i8", 10, 1000, 256), ("i8", 10, 1000, 4096), ("i4", 64, 512, 1000), ("i2", 33, 2048, 513),
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
@@ -389,11 +393,11 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
 
 
 @pytest.mark.parametrize("fmt,N,K,n", [
-    # K not a multiple of 64 keeps a layer on the single-stage tiled GEMM; by tile count it runs 64 x 64,
-    # 64 x 128 or 128 x 128 tiles (ragged edges in both directions), rows that are not whole 16-byte units take
-    # the element-wise loads and always 64 x 64
-    ("bf16", 512, 784, 600), ("i8", 1000, 528, 4096), ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096),
-    ("i4", 520, 1056, 300), ("i2", 2048, 1056, 2048),
+    # Too few 256 x 256 tiles and too few K tiles to split K over the grid: the single-stage tiled GEMM; by tile
+    # count it runs 64 x 64, 64 x 128 or 128 x 128 tiles (ragged edges in both directions), rows that are not whole
+    # 16-byte units take the element-wise loads and always 64 x 64
+    ("bf16", 512, 784, 600), ("i8", 1000, 528, 4096),
+    ("i2", 2048, 1056, 2048),
     ("i8", 300, 1000, 700), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 512),
     # integer rows that are whole 32-bit words but not whole 16-byte units (784 INT4 codes = 392 bytes): word loads
     ("i4", 512, 784, 1024), ("i2", 300, 784, 300), ("i8", 1000, 776, 600), ("i4", 520, 1000, 64), ("i2", 2048, 1008, 2048),
@@ -406,6 +410,26 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     want = np.where(pre > 0, pre, 0.01 * pre)
     got = net.forward(X)
     assert _kernel_of(S, net, n) == "sp_gemm16"
+    assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
+    net.destroy()
+
+
+@pytest.mark.parametrize("fmt,N,K,n", [
+    # K not a multiple of 64 with 16-byte rows: the 256 x 256 tile kernel takes the partial K tile first.
+    # Enough tiles for the chip (tails of 40, 8, 48 and 32 elements) ...
+    ("bf16", 4096, 1000, 4096), ("f16", 4096, 1096, 3000), ("i8", 4096, 1008, 4096), ("i4", 4096, 1056, 4096),
+    # ... K split over the grid, the partial tile in the last split ...
+    ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096), ("i4", 520, 1056, 300), ("i8", 1100, 2000, 700),
+    # ... a single row of 128 x 256 tiles, ragged in M and N, and a K of two tiles and a bit
+    ("bf16", 8192, 1000, 100), ("f16", 5000, 1160, 77), ("bf16", 8200, 136, 8200),
+])
+def test_big_tile_gemm_takes_a_partial_k_tile(S, fmt, N, K, n):
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
+    X = np.random.default_rng(n + 1).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert _kernel_of(S, net, n) == "sp_gemm16_big"
     assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
     net.destroy()
 
