@@ -245,12 +245,13 @@ __device__ __forceinline__ float apply_act_cheap(float x, int act)
     }
 }
 
+// FP32 -> BF16, round to nearest even, NaNs stay NaNs: the part's own conversion instruction
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x)
 {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    const __bf16 h = (__bf16)x;
+    uint16_t r;
+    __builtin_memcpy(&r, &h, 2);
+    return r;
 }
 
 // FP32 -> FP16: finite values beyond the FP16 range become +-65504 (an activation that large stays finite in the

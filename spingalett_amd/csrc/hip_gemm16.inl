@@ -290,26 +290,33 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
         }
     }
 
-    // epilogue: scale, bias, activation, store
+    // epilogue: scale, bias, activation, store.  Sigmoid and tanh have a copy of the loops to themselves: a switch
+    // over all activations behind every one of a lane's outputs is mostly their code, fetched for nothing.
     const float wscale = g.L.wscale;
+    auto emit = [&](auto slow_c) __attribute__((always_inline)) {
+        constexpr bool SLOW = decltype(slow_c)::value;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
-        if (col >= N) continue;
-        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+            if (col >= N) continue;
+            const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+            for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t row = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row >= M) continue;
-                const float v = apply_act(fmaf(acc[i][j][r], wscale, bias), g.L.act);
-                const size_t o = (size_t)row * N + col;
-                if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
-                else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row >= M) continue;
+                    const float pre = fmaf(acc[i][j][r], wscale, bias);
+                    const float v = SLOW ? apply_act(pre, g.L.act) : apply_act_cheap(pre, g.L.act);
+                    const size_t o = (size_t)row * N + col;
+                    if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+                    else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+                }
             }
         }
-    }
+    };
+    if (g.L.act == A_SIGMOID || g.L.act == A_TANH) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 template <int OFF>
@@ -383,35 +390,26 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave / WN, wn = wave % WN;
 
-    // tile order: each XCD (workgroup id mod 8) gets a contiguous run of tiles; inside
-    // the run, 8 row tiles x 4 column tiles are consecutive so that the 32 workgroups
-    // an XCD runs at once share A rows and W rows in its L2
+    // Tile order: each XCD (workgroup id mod 8) gets a contiguous run of tiles; inside the run, 8 row tiles x 4
+    // column tiles are consecutive so that the 32 workgroups an XCD runs at once share A rows and W rows in its L2.
+    // (A workgroup that walks over several tiles instead, one workgroup per compute unit, was measured: no faster,
+    // and the longer live ranges cost the integer formats register spills.)
     const uint32_t tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
     const uint32_t ntiles = tiles_m * tiles_n;
-    uint32_t bid = blockIdx.x;
-    {
+    uint32_t m0 = 0, n0 = 0;
+    auto place = [&](uint32_t bid) {
         const uint32_t per = ntiles / 8u;
         if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
-    }
-    uint32_t tm, tn;
-    {
         constexpr uint32_t GM = 8;
         const uint32_t group = bid / (GM * tiles_n);
         const uint32_t first = group * GM;
         const uint32_t rows = tiles_m - first < GM ? tiles_m - first : GM;
         const uint32_t in = bid - group * GM * tiles_n;
-        tm = first + in % rows;
-        tn = in / rows;
-    }
-    const uint32_t m0 = tm * BM, n0 = tn * BN;
+        m0 = (first + in % rows) * BM;
+        n0 = (in / rows) * BN;
+    };
 
     f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     // LDS-DMA sources: a uniform base (advanced per K tile on the scalar unit) plus a fixed 32-bit
     // byte offset per lane and issue, and LDS destinations derived from a scalar wave index: the main
@@ -426,22 +424,24 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     constexpr int PER = NWAVES / HALF;                            // shares a loader wave issues
     constexpr int A_DUTY = PER * A_ISSUES, W_DUTY = W_DIRECT ? PER * W_ISSUES : 1;
     uint32_t a_voff[A_DUTY], w_voff[W_DUTY];
+    auto lane_offsets = [&]() {
 #pragma unroll
-    for (int d = 0; d < A_DUTY; ++d) {
-        const int i = d / PER, wv = (wave & (HALF - 1)) + (d % PER) * HALF;
-        const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
-        const uint32_t m = m0 + row < M ? m0 + row : M - 1;
-        a_voff[d] = (uint32_t)(((size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
-    }
-    if constexpr (W_DIRECT) {
-#pragma unroll
-        for (int d = 0; d < W_DUTY; ++d) {
+        for (int d = 0; d < A_DUTY; ++d) {
             const int i = d / PER, wv = (wave & (HALF - 1)) + (d % PER) * HALF;
             const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
-            const uint32_t n = n0 + row < N ? n0 + row : N - 1;
-            w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
+            const uint32_t m = m0 + row < M ? m0 + row : M - 1;
+            a_voff[d] = (uint32_t)(((size_t)m * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
         }
-    }
+        if constexpr (W_DIRECT) {
+#pragma unroll
+            for (int d = 0; d < W_DUTY; ++d) {
+                const int i = d / PER, wv = (wave & (HALF - 1)) + (d % PER) * HALF;
+                const int ci = (i * NWAVES + wv) * 64 + lane, row = ci >> 3, pos = ci & 7;
+                const uint32_t n = n0 + row < N ? n0 + row : N - 1;
+                w_voff[d] = (uint32_t)(((size_t)n * K + ((pos ^ ((row >> 1) & 7)) << 3)) * 2u);
+            }
+        }
+    };
     // which 8 elements of a 64-element tile row this lane fetches: the same for every load it issues, because
     // the rows of two of its loads are a multiple of 16 apart
     static_assert(NWAVES % 2 == 0 && HALF % 2 == 0, "the swizzle of a lane's loads must not depend on the load");
@@ -627,6 +627,14 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     const uint32_t tail = (kend - kbeg) % BK;              // only the last K split can have one
     // tile 0 is the partial tile if there is one; tile s >= 1 then starts at kbeg + (s - 1) * BK
     const uint32_t kshift = tail ? (uint32_t)BK : 0u;
+    place(blockIdx.x);
+    lane_offsets();
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     if (tail) {
         const uint32_t kt0 = kend - tail;
         issue_tail(kt0);
@@ -677,6 +685,10 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
         // unrolled loops puts a copy of their code behind each of a lane's 16 TM TN outputs, and fetching that code
         // took longer than the stores (a tenth of an 8192-cubed launch).  The lambda is forced inline: called, it
         // would take the accumulators through memory.
+        // Long K: the outputs bypass the caches' usual retention (they would displace the A and W panels the other
+        // tiles of the die are re-reading: 8192 cubed 0.908 against 0.934 ms); short K: the next layer reads them
+        // back soon and they are most of the traffic (8192 x 8192 x 1024: 0.162 against 0.175 ms the other way round).
+        const bool stream_out = K >= 2048u;
         auto turn = [&](auto es_c, auto slow_c) __attribute__((always_inline)) {
             constexpr int ES = decltype(es_c)::value;
             constexpr bool SLOW = decltype(slow_c)::value;
@@ -703,9 +715,12 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
                     const uint4 v = *reinterpret_cast<const uint4 *>(mine + rl * PITCH + seg * 16);
                     const uint32_t row = m0 + (wm * TM + i) * 32 + rl;
                     const uint32_t col = n0 + wn * BW + seg * (16 / ES);
-                    if (row < M && col < N)                          // N is a multiple of 16 / ES: a unit is all in or all out
-                        __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w},
-                                                    reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(g.C) + ((size_t)row * N + col) * ES));
+                    if (row < M && col < N) {                        // N is a multiple of 16 / ES: a unit is all in or all out
+                        u32x4 *dstp = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(g.C) + ((size_t)row * N + col) * ES);
+                        const u32x4 vv{v.x, v.y, v.z, v.w};
+                        if (stream_out) __builtin_nontemporal_store(vv, dstp);
+                        else *dstp = vv;
+                    }
                 }
             }
         };

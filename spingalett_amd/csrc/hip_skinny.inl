@@ -121,15 +121,24 @@ __device__ __forceinline__ void skinny_frag(const uint4 &v, int j, uint32_t (&f)
     }
 }
 
-template <bool F16T>
-__device__ __forceinline__ void skinny_emit(const SkinnyArgs &a, uint32_t c, uint32_t r, float accv)
+// SLOW: the activation may be sigmoid or tanh.  Callers with many outputs per lane keep a copy of their loops for
+// those two: a switch over all activations behind every output is mostly their code, fetched for nothing.
+template <bool F16T, bool SLOW = true>
+__device__ __forceinline__ void skinny_emit_biased(const SkinnyArgs &a, uint32_t c, uint32_t r, float accv, float bias)
 {
     const uint32_t m = a.mode_b ? r : c, n = a.mode_b ? c : r;
-    const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, n) * a.L.bscale;
-    const float v = apply_act(fmaf(accv, a.L.wscale, bias), a.L.act);
+    const float pre = fmaf(accv, a.L.wscale, bias);
+    const float v = SLOW ? apply_act(pre, a.L.act) : apply_act_cheap(pre, a.L.act);
     const size_t o = (size_t)m * a.L.N + n;
     if (a.out_f32) reinterpret_cast<float *>(a.C)[o] = v;
     else reinterpret_cast<uint16_t *>(a.C)[o] = f32_to_t16<F16T>(v);
+}
+
+template <bool F16T>
+__device__ __forceinline__ void skinny_emit(const SkinnyArgs &a, uint32_t c, uint32_t r, float accv)
+{
+    const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, a.mode_b ? c : r) * a.L.bscale;
+    skinny_emit_biased<F16T>(a, c, r, accv, bias);
 }
 
 // 16 bytes per lane from scalar base + 32-bit lane offset + immediate.  Inline assembly: the compiler's
@@ -351,20 +360,42 @@ __global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the redundant tail loads
 
     // accumulator register r of lane (n31, h): thin row 8 (r / 4) + 4 h + r % 4, streamed row n31
+    if (a.ws) {
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        const uint32_t r = row0 + rt * 32u + n31;
-        if (r >= a.R) continue;
+        for (int rt = 0; rt < RT; ++rt) {
+            const uint32_t r = row0 + rt * 32u + n31;
+            if (r >= a.R) continue;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+            for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                const uint32_t c = cbase + ct * 32u + 8u * (q >> 2) + 4u * h + (q & 3);
-                if (c >= a.NC) continue;
-                if (a.ws) a.ws[((size_t)blockIdx.y * a.NC + c) * a.R + r] = acc[rt][ct][q];
-                else skinny_emit<F16T>(a, c, r, acc[rt][ct][q]);
-            }
+                for (int q = 0; q < 16; ++q) {
+                    const uint32_t c = cbase + ct * 32u + 8u * (q >> 2) + 4u * h + (q & 3);
+                    if (c < a.NC) a.ws[((size_t)blockIdx.y * a.NC + c) * a.R + r] = acc[rt][ct][q];
+                }
+        }
+        return;
     }
+    auto emit = [&](auto slow_c) __attribute__((always_inline)) {
+        constexpr bool SLOW = decltype(slow_c)::value;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const uint32_t r = row0 + rt * 32u + n31;
+            if (r >= a.R) continue;
+            // streamed rows that are outputs have one bias per lane and row tile
+            const float bias_r = a.mode_b ? 0.0f : elem_value_rt(a.L.bias_fmt, a.L.bias, r) * a.L.bscale;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    const uint32_t c = cbase + ct * 32u + 8u * (q >> 2) + 4u * h + (q & 3);
+                    if (c >= a.NC) continue;
+                    const float bias = a.mode_b ? elem_value_rt(a.L.bias_fmt, a.L.bias, c) * a.L.bscale : bias_r;
+                    skinny_emit_biased<F16T, SLOW>(a, c, r, acc[rt][ct][q], bias);
+                }
+        }
+    };
+    if (a.L.act == A_SIGMOID || a.L.act == A_TANH) emit(std::true_type{});
+    else emit(std::false_type{});
 }
 
 // Variant for a thin operand of at most NCP (8 or 16; the host uses 8) rows: the NW waves of a workgroup share one tile of 32
