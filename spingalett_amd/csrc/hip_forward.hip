@@ -1037,7 +1037,12 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
             (void)once;
             kern<<<grid, 512, lds, g_stream>>>(g);
         }
-        if (g.ws) sp_gemm16_reduce<F16T><<<(uint32_t)(((uint64_t)M * L.N + 255) / 256), 256, 0, g_stream>>>(g, splits);
+        if (g.ws) {
+            const uint64_t total = (uint64_t)M * L.N;
+            const bool vec = L.N % 4u == 0 && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+            if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, splits);
+            else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, splits);
+        }
         return;
     }
     g.kper = 0;

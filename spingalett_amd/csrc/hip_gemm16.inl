@@ -653,7 +653,8 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
         stage(std::integral_constant<int, 0>{}, kt + 1 < ktiles, kbeg + (kt + 1) * BK - kshift);
         if (kt + 1 < ktiles) stage(std::integral_constant<int, 1>{}, kt + 2 < ktiles, kbeg + (kt + 2) * BK - kshift);
     }
-    if (g.ws) {
+    // partial sums of a K split whose rows are not whole 16-byte units: one element per lane and store
+    if (g.ws && (N % 4u != 0 || (reinterpret_cast<uintptr_t>(g.ws) & 15u) != 0)) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
@@ -672,15 +673,17 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     // Output rows that are whole 16-byte units: a wave turns its 32 x (32 TN) block of each row tile around in LDS
     // (the stages are free after the loop's last barrier; every wave has a region of its own, so no barrier is
     // needed) and writes whole rows of the block, 16 bytes per lane, instead of one element per lane.
+    // The partial sums of a K split go the same way into the workspace, unscaled, as FP32.
     const uint32_t esz = g.out_f32 ? 4u : 2u;
-    if (((size_t)N * esz) % 16u == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0) {
+    if (g.ws || (((size_t)N * esz) % 16u == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0)) {
         constexpr int BW = 32 * TN;                                  // columns of a wave's block
         float bias[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31);
-            bias[j] = col < N ? elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale : 0.0f;
+            bias[j] = (col < N && !g.ws) ? elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale : 0.0f;
         }
+        char *const out = g.ws ? reinterpret_cast<char *>(g.ws + (size_t)blockIdx.y * M * N) : reinterpret_cast<char *>(g.C);
         // Sigmoid and tanh are kept out of the common path: a run-time switch over all activations inside the
         // unrolled loops puts a copy of their code behind each of a lane's 16 TM TN outputs, and fetching that code
         // took longer than the stores (a tenth of an 8192-cubed launch).  The lambda is forced inline: called, it
@@ -688,10 +691,10 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
         // Long K: the outputs bypass the caches' usual retention (they would displace the A and W panels the other
         // tiles of the die are re-reading: 8192 cubed 0.908 against 0.934 ms); short K: the next layer reads them
         // back soon and they are most of the traffic (8192 x 8192 x 1024: 0.162 against 0.175 ms the other way round).
-        const bool stream_out = K >= 2048u;
-        auto turn = [&](auto es_c, auto slow_c) __attribute__((always_inline)) {
+        const bool stream_out = K >= 2048u && !g.ws;
+        auto turn = [&](auto es_c, auto mode_c) __attribute__((always_inline)) {
             constexpr int ES = decltype(es_c)::value;
-            constexpr bool SLOW = decltype(slow_c)::value;
+            constexpr int MODE = decltype(mode_c)::value;            // 0: cheap activations, 1: sigmoid / tanh, 2: partial sums
             constexpr int PITCH = BW * ES + 16;                      // lanes 0-31 and 32-63 (four rows apart) on different banks
             constexpr int LPR = BW * ES / 16;                        // lanes that write one row
             constexpr int RPP = 64 / LPR;                            // rows per store instruction
@@ -703,8 +706,8 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int rl = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                        const float pre = fmaf(acc[i][j][r], wscale, bias[j]);
-                        const float v = SLOW ? apply_act(pre, g.L.act) : apply_act_cheap(pre, g.L.act);
+                        const float pre = MODE == 2 ? acc[i][j][r] : fmaf(acc[i][j][r], wscale, bias[j]);
+                        const float v = MODE == 2 ? pre : MODE == 1 ? apply_act(pre, g.L.act) : apply_act_cheap(pre, g.L.act);
                         char *dst = mine + rl * PITCH + (j * 32 + (lane & 31)) * ES;
                         if constexpr (ES == 4) *reinterpret_cast<float *>(dst) = v;
                         else *reinterpret_cast<uint16_t *>(dst) = f32_to_t16<F16T>(v);
@@ -716,7 +719,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
                     const uint32_t row = m0 + (wm * TM + i) * 32 + rl;
                     const uint32_t col = n0 + wn * BW + seg * (16 / ES);
                     if (row < M && col < N) {                        // N is a multiple of 16 / ES: a unit is all in or all out
-                        u32x4 *dstp = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(g.C) + ((size_t)row * N + col) * ES);
+                        u32x4 *dstp = reinterpret_cast<u32x4 *>(out + ((size_t)row * N + col) * ES);
                         const u32x4 vv{v.x, v.y, v.z, v.w};
                         if (stream_out) __builtin_nontemporal_store(vv, dstp);
                         else *dstp = vv;
@@ -725,12 +728,16 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
             }
         };
         const bool slow = g.L.act == A_SIGMOID || g.L.act == A_TANH;
-        if (g.out_f32) {
-            if (slow) turn(std::integral_constant<int, 4>{}, std::true_type{});
-            else turn(std::integral_constant<int, 4>{}, std::false_type{});
+        using E4 = std::integral_constant<int, 4>;
+        using E2 = std::integral_constant<int, 2>;
+        if (g.ws) {
+            turn(E4{}, std::integral_constant<int, 2>{});
+        } else if (g.out_f32) {
+            if (slow) turn(E4{}, std::integral_constant<int, 1>{});
+            else turn(E4{}, std::integral_constant<int, 0>{});
         } else {
-            if (slow) turn(std::integral_constant<int, 2>{}, std::true_type{});
-            else turn(std::integral_constant<int, 2>{}, std::false_type{});
+            if (slow) turn(E2{}, std::integral_constant<int, 1>{});
+            else turn(E2{}, std::integral_constant<int, 0>{});
         }
         return;
     }
@@ -755,17 +762,44 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
 }
 
 // adds the K splits of sp_gemm16_big (in split order) and applies scale, bias and activation
-template <bool F16T>
+// adds the K splits of sp_gemm16_big and applies scale, bias and activation; a thread takes four neighbouring
+// columns (VEC: N a multiple of four, workspace and C 16-byte aligned) or one
+template <bool F16T, bool VEC>
 __global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32_t splits)
 {
-    const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
     const uint64_t total = (uint64_t)g.M * g.L.N;
-    if (idx >= total) return;
-    float sum = 0.0f;
-    for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
-    const uint32_t col = (uint32_t)(idx % g.L.N);
-    const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
-    const float v = apply_act(fmaf(sum, g.L.wscale, bias), g.L.act);
-    if (g.out_f32) reinterpret_cast<float *>(g.C)[idx] = v;
-    else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
+    if constexpr (VEC) {
+        const uint64_t idx = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+        if (idx >= total) return;
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (uint32_t sp = 0; sp < splits; ++sp) {
+            const float4 v = *reinterpret_cast<const float4 *>(g.ws + (uint64_t)sp * total + idx);
+            sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+        }
+        const uint32_t col = (uint32_t)(idx % g.L.N);
+        const float in[4] = {sum.x, sum.y, sum.z, sum.w};
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col + i) * g.L.bscale;
+            v[i] = apply_act(fmaf(in[i], g.L.wscale, bias), g.L.act);
+        }
+        if (g.out_f32) {
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(g.C) + idx) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            const uint32_t lo = (uint32_t)f32_to_t16<F16T>(v[0]) | ((uint32_t)f32_to_t16<F16T>(v[1]) << 16);
+            const uint32_t hi = (uint32_t)f32_to_t16<F16T>(v[2]) | ((uint32_t)f32_to_t16<F16T>(v[3]) << 16);
+            *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(g.C) + idx) = make_uint2(lo, hi);
+        }
+    } else {
+        const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+        if (idx >= total) return;
+        float sum = 0.0f;
+        for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
+        const uint32_t col = (uint32_t)(idx % g.L.N);
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+        const float v = apply_act(fmaf(sum, g.L.wscale, bias), g.L.act);
+        if (g.out_f32) reinterpret_cast<float *>(g.C)[idx] = v;
+        else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
+    }
 }
