@@ -62,7 +62,7 @@ def compute_dtype(prec: int, n: int) -> str:
         return "f32"
     if n <= 4:
         return "i8 (exact integer digits, f32 accumulate)" if prec >= S.PRECISION_INT8 else "f32"
-    return "bf16" if prec == S.PRECISION_BFLOAT16 else "f16"
+    return "f16"         # FP16 matrix cores, f32 accumulate (BF16 weights: against their FP16 copy)
 
 
 def array_payload(n: int, prec: int) -> int:
@@ -148,14 +148,14 @@ def device_copies(net, topo, prec, min_total_bytes: int):
     return copies, clones
 
 
-def time_workload(copies, topo, n, x_host, steps, warmup):
+def time_workload(copies, topo, n, x_host, steps, warmup, flags=0):
     d_x = S.DeviceBuffer.from_numpy(x_host)
     d_y = S.DeviceBuffer(4 * n * topo[-1])
     if warmup > 0:
-        S.time_forward(copies, d_x, n, d_y, warmup)
+        S.time_forward(copies, d_x, n, d_y, warmup, flags)
     S.synchronize()
     t0 = time.perf_counter()
-    ev_ms = S.time_forward(copies, d_x, n, d_y, steps)      # records events, waits for the last one
+    ev_ms = S.time_forward(copies, d_x, n, d_y, steps, flags)      # records events, waits for the last one
     S.synchronize()
     wall = time.perf_counter() - t0
     y = d_y.to_numpy(np.float32, (n, topo[-1]))
@@ -187,11 +187,18 @@ def dominant_layer(topo):
     return 1 + int(np.argmax([topo[l] * topo[l + 1] for l in range(len(topo) - 1)]))
 
 
+def timed_layer(copies, l, n, iters, flags=0):
+    """Average milliseconds of layer l's launches, back to back, after enough of them to bring the part to the clocks
+    it holds under this load (about 50 ms: the first launches after a pause on the host run 5-10 % slower)."""
+    first = S.time_layer(copies, l, n, len(copies) + 2, flags) / (len(copies) + 2)
+    S.time_layer(copies, l, n, int(min(2000, max(3, 50.0 / max(first, 1e-3)))), flags)
+    return S.time_layer(copies, l, n, iters, flags) / iters
+
+
 def roofline_for(copies, topo, prec, n, iters):
     """Times the main kernel of the largest layer alone (HIP events on its stream)."""
     l = dominant_layer(topo)
-    S.time_layer(copies, l, n, len(copies) + 2)
-    ms = S.time_layer(copies, l, n, iters) / iters
+    ms = timed_layer(copies, l, n, iters)
     K, N = topo[l - 1], topo[l]
     kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
     traffic = PROFILED_TRAFFIC.get((kernel, (n, N, K)))
@@ -251,6 +258,17 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
                    mfma_frac=fl / (ms_ev * 1e-3) / (FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK),
                    copies=len(copies), finite=bool(np.isfinite(y).all()))
         row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
+        if prec == S.PRECISION_BFLOAT16 and n >= 5:
+            # the same workload with BF16 activations on the BF16 matrix cores (SPHIP_BF16_ACTIVATIONS /
+            # spingalett_set_bf16_activations): the faster, less accurate setting; the figures above are the default's
+            # (FP16 activations against the FP16 copy of the BF16 weights)
+            alt = S.SPHIP_BF16_ACTIVATIONS
+            w_wall, w_ev, _ = time_workload(copies, topo, n, x, k, warmup, alt)
+            l = dominant_layer(topo)
+            w_layer = timed_layer(copies, l, n, 20, alt)
+            row["bf16_activations"] = dict(ms_per_step=w_wall, samples_per_s=n / (w_wall * 1e-3),
+                                           mfma_frac=fl / (w_ev * 1e-3) / MFMA16_PEAK, dominant_layer_ms=w_layer,
+                                           dominant_layer_frac=2.0 * n * topo[l - 1] * topo[l] / (w_layer * 1e-3) / MFMA16_PEAK)
         if n == 1:
             # the public forward(): host pointer in, all activations mirrored into net->neurons (PCIe both ways)
             x1 = np.ascontiguousarray(x[0])
@@ -432,6 +450,7 @@ def main():
         "roofline": {k: rl[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
         "roofline_kernel": {k: rl[k] for k in ("kernel", "layer", "shape", "avg_ms")},
         "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
+        "bf16_activations": row.get("bf16_activations"),
         "cpu_baseline": cpu,
         "workloads": extra,
         "training": training,

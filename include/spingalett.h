@@ -267,6 +267,17 @@ typedef enum { SPINGALETT_DEQUANT_STRICT, SPINGALETT_DEQUANT_RELEASE } Spingalet
 SPINGALETT_API void spingalett_set_dequant_mode(SpingalettDequantMode mode);
 SPINGALETT_API SpingalettDequantMode spingalett_get_dequant_mode(void);
 
+/* Activation type between the layers of a BF16 net on the matrix-core path (5 samples and more; the reference keeps
+ * FP32 activations, Training.c:313-345):
+ *   FP16 — FP16 activations (11 significant bits) on the FP16 matrix cores, against an FP16 copy of the weights that
+ *          is made when they reach the device (twice the weight memory); the default.
+ *   BF16 — BF16 activations (8 bits) on the BF16 matrix cores: a few per cent faster, further from the reference's
+ *          outputs.
+ * Other weight formats always run FP16 activations (integer and FP16 weights) or FP32 arithmetic (FP32 weights). */
+typedef enum { SPINGALETT_BF16_ACTIVATIONS_FP16, SPINGALETT_BF16_ACTIVATIONS_BF16 } SpingalettBf16Activations;
+SPINGALETT_API void spingalett_set_bf16_activations(SpingalettBf16Activations mode);
+SPINGALETT_API SpingalettBf16Activations spingalett_get_bf16_activations(void);
+
 /* Batched forward: the public form of the reference's static
  * batch_forward(net, ws, inputs, N) (Training.c:313-345).  inputs is
  * row-major [n][topology[0]], outputs row-major [n][topology[last]], both

@@ -42,6 +42,12 @@ typedef struct {
 #define SPHIP_TRAIN_SAME_BATCH 4u /* sphip_train_step: reuse the host batch the previous step copied in */
 #define SPHIP_FORCE_GEMM    8u   /* use the matrix-core path whatever n is      */
 #define SPHIP_FORCE_GEMV   16u   /* use the vector path (n <= 64)               */
+/* BF16 weights on the matrix-core path (5 samples and more) are multiplied with FP16 activations on the FP16 matrix
+ * cores, against an FP16 copy of each weight array that sphip_upload_array makes (the weights times a power of two
+ * that brings them into FP16's range: as many bytes again).  This flag selects BF16 activations on the BF16 matrix
+ * cores instead: 8 instead of 11 significant bits between layers, a few per cent faster.  Other formats and the
+ * vector path ignore it; no counterpart in the reference, whose activations are FP32. */
+#define SPHIP_BF16_ACTIVATIONS 32u
 
 SPHIP_API int  sphip_device_count(void);
 SPHIP_API const char *sphip_last_error_string(void);   /* per thread */
@@ -78,7 +84,7 @@ SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *
  * A batch whose workspace exceeds the array is refused with an error that names both sizes (sphip_forward takes it).
  * Nothing in the array needs clearing between calls: every kernel reads only what this call wrote.  All calls on one
  * GPU share the array, so two calls that overlap in time (from different threads) race; nets of more than 64 layers
- * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV only. */
+ * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV / SPHIP_BF16_ACTIVATIONS only. */
 #define SPHIP_NOALLOC_SCRATCH_BYTES (64u << 20)
 SPHIP_API int  sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags);
 /* The evaluation step that follows batch_forward in the reference's epoch loop, on the device:

@@ -95,6 +95,12 @@ static bool ensure_device(sp_net *sn)
     return true;
 }
 
+/* what spingalett_set_bf16_activations asks of the batched entry points */
+static uint32_t activation_flags(void)
+{
+    return spingalett_get_bf16_activations() == SPINGALETT_BF16_ACTIVATIONS_BF16 ? SPHIP_BF16_ACTIVATIONS : 0u;
+}
+
 static sp_net *checked(NeuralNetwork *net, const char *who)
 {
     if (!net) {
@@ -133,7 +139,7 @@ float *spingalett_forward_batch(NeuralNetwork *net, const float *inputs, uint32_
     if (!sn) return NULL;
     if (n == 0) return outputs;
     if (!ensure_device(sn)) return NULL;
-    if (sphip_forward(sn->dev, inputs, n, outputs, 0)) {
+    if (sphip_forward(sn->dev, inputs, n, outputs, activation_flags())) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: forward_batch");
         return NULL;
     }
@@ -149,7 +155,7 @@ int spingalett_forward_batch_device(NeuralNetwork *net, const float *d_inputs, u
         return 1;
     }
     if (!ensure_device(sn)) return 1;
-    if (sphip_forward(sn->dev, d_inputs, n, d_outputs, SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE)) {
+    if (sphip_forward(sn->dev, d_inputs, n, d_outputs, SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE | activation_flags())) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: forward_batch_device");
         return 1;
     }
@@ -171,7 +177,7 @@ int spingalett_evaluate_batch(NeuralNetwork *net, const float *inputs, const flo
         return 1;
     }
     if (!ensure_device(sn)) return 1;
-    if (sphip_evaluate(sn->dev, inputs, targets, n, (int)net->loss_func, 0, total_loss, predictions, correct)) {
+    if (sphip_evaluate(sn->dev, inputs, targets, n, (int)net->loss_func, activation_flags(), total_loss, predictions, correct)) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: evaluate_batch");
         return 1;
     }

@@ -424,6 +424,30 @@ __global__ __launch_bounds__(256) void sp_cvt16(const float *__restrict__ in, ui
     }
 }
 
+// largest bit pattern of |w| among the finite BF16 values of an array
+__global__ __launch_bounds__(256) void sp_absmax_bf16(const uint16_t *__restrict__ w, uint64_t n, uint32_t *__restrict__ out)
+{
+    uint32_t m = 0;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256u) {
+        const uint32_t a = w[i] & 0x7FFFu;
+        if (a < 0x7F80u && a > m) m = a;
+    }
+    for (int off = 32; off; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
+}
+
+// BF16 -> FP16 of w * 2^shift (the shift puts the array's largest magnitude just below FP16's largest power of two,
+// so only values 2^-29 of it and smaller leave the normal range); round to nearest even, exact for every value whose
+// scaled magnitude is at least 2^-14, since BF16 has fewer significant bits than FP16
+__global__ __launch_bounds__(256) void sp_bf16_to_f16(const uint16_t *__restrict__ w, uint16_t *__restrict__ out, uint64_t n, int shift)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) out[i] = f32_to_f16_sat(ldexpf(__uint_as_float((uint32_t)w[i] << 16), shift));
+}
+
 #include "hip_gemm16.inl"
 
 #include "hip_skinny.inl"
@@ -547,6 +571,9 @@ struct DevArray {
     bool uploaded = false;
     uint16_t *codes16 = nullptr;   // weights of a layer with few outputs: unscaled codes as FP16 (made on demand)
     bool codes16_valid = false;
+    uint16_t *wide16 = nullptr;    // BF16 weight arrays: the weights times 2^wide_shift as FP16 (made at upload)
+    bool wide16_valid = false;
+    int wide_shift = 0;
 };
 
 struct sphip_train_state;
@@ -1252,7 +1279,9 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
                     uint32_t only_layer, bool keep = false)
 {
     const Regime reg = pick_regime(net, n, flags);
-    const bool f16t = net->prec != BF16;          // 16-bit activation type of the matrix-core path
+    // BF16 weights: FP16 activations against the FP16 copy of the weights unless BF16 activations are asked for
+    const bool wide = !(flags & SPHIP_BF16_ACTIVATIONS) && net->prec == BF16 && reg == R_GEMM16;
+    const bool f16t = net->prec != BF16 || wide;  // 16-bit activation type of the matrix-core path
     const uint32_t last = net->layers - 1;
 
     const void *in = d_x;
@@ -1267,7 +1296,11 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
     }
 
     for (uint32_t l = 1; l <= last; ++l) {
-        const LayerArgs L = make_layer_args(net, l);
+        LayerArgs L = make_layer_args(net, l);
+        if (wide) {
+            L.w = reinterpret_cast<const uint8_t *>(net->W[l - 1].wide16);
+            L.wscale = ldexpf(L.wscale, -net->W[l - 1].wide_shift);
+        }
         const bool softmax = net->act[l - 1] == A_SOFTMAX;
         const bool is_last = l == last;
         void *dst = is_last ? (void *)d_y : keep ? (void *)(net->layers_buf + net->slot_off[l]) : wk.buf[(l + 1) & 1];
@@ -1285,7 +1318,8 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
             else {
                 const DevArray &wa = net->W[l - 1];
                 ThinCtx ctx{};
-                if (net->prec == F16 || net->prec == BF16) ctx.w16 = reinterpret_cast<const uint16_t *>(wa.base);
+                if (wide) ctx.w16 = wa.wide16;
+                else if (net->prec == F16 || net->prec == BF16) ctx.w16 = reinterpret_cast<const uint16_t *>(wa.base);
                 else ctx.w16 = wk.codes16[l - 1];
                 ctx.ws = wk.split_ws;
                 ctx.ws_floats = wk.split_cap;
@@ -1294,7 +1328,7 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
                     ctx.soft_kind = !is_last ? (f16t ? 2 : 1) : 0;
                     ctx.soft_done = &soft_done;
                 }
-                launch_gemm16(net->prec, L, (const uint16_t *)in, main_out, n, out_f32, ctx);
+                launch_gemm16(wide ? (int)F16 : net->prec, L, (const uint16_t *)in, main_out, n, out_f32, ctx);
             }
         }
         if (softmax && !only_layer && !soft_done) {
@@ -1365,7 +1399,7 @@ void sphip_destroy(sphip_net *net)
     if (!net) return;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
     train_free(net);
-    for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); }
+    for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); if (a.wide16) (void)hipFree(a.wide16); }
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
     if (net->split_ws) (void)hipFree(net->split_ws);
     if (net->eval_buf) (void)hipFree(net->eval_buf);
@@ -1382,6 +1416,30 @@ void sphip_destroy(sphip_net *net)
     delete net;
 }
 
+// A BF16 weight array's FP16 copy for the matrix-core path with FP16 activations: the weights times the power of
+// two that brings the array's largest magnitude into [2^14, 2^15).  One small reduction, one wait, one conversion.
+uint32_t *g_absmax_word = nullptr;
+
+int make_wide(DevArray &wa)
+{
+    if (!g_absmax_word) HCHECK(hipMalloc((void **)&g_absmax_word, sizeof(uint32_t)));
+    if (!wa.wide16) HCHECK(hipMalloc((void **)&wa.wide16, wa.count * sizeof(uint16_t)));
+    const uint16_t *src = reinterpret_cast<const uint16_t *>(wa.base);
+    uint32_t top = 0;
+    HCHECK(hipMemsetAsync(g_absmax_word, 0, sizeof(uint32_t), g_stream));
+    uint64_t blocks = (wa.count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    sp_absmax_bf16<<<(uint32_t)blocks, 256, 0, g_stream>>>(src, wa.count, g_absmax_word);
+    HCHECK(hipMemcpyAsync(&top, g_absmax_word, sizeof(uint32_t), hipMemcpyDeviceToHost, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    wa.wide_shift = top ? 14 - ((int)(top >> 7) - 127) : 0;       // largest magnitude = 1.m x 2^(e - 127)
+    sp_bf16_to_f16<<<(uint32_t)((wa.count + 255) / 256), 256, 0, g_stream>>>(src, wa.wide16, wa.count, wa.wide_shift);
+    HCHECK(hipGetLastError());
+    HCHECK(hipStreamSynchronize(g_stream));
+    wa.wide16_valid = true;
+    return 0;
+}
+
 int sphip_upload_array(sphip_net *net, uint32_t l, int which, const void *codes, size_t bytes, float max_val)
 {
     if (!net || l + 1 >= net->layers || (which != 0 && which != 1) || !codes) return fail_msg("sphip_upload_array: invalid argument");
@@ -1392,6 +1450,8 @@ int sphip_upload_array(sphip_net *net, uint32_t l, int which, const void *codes,
     a.max_val = max_val;
     a.uploaded = true;
     a.codes16_valid = false;
+    a.wide16_valid = false;
+    if (which == 0 && net->prec == BF16 && make_wide(a)) return 1;
     return 0;
 }
 
@@ -1409,6 +1469,13 @@ int sphip_clone(const sphip_net *src, sphip_net **out)
             if (e != hipSuccess) { sphip_destroy(net); return fail_hip("sphip_clone copy", e); }
             t.max_val = s.max_val;
             t.uploaded = s.uploaded;
+            if (s.wide16_valid) {
+                e = hipMalloc((void **)&t.wide16, s.count * sizeof(uint16_t));
+                if (e == hipSuccess) e = hipMemcpyAsync(t.wide16, s.wide16, s.count * sizeof(uint16_t), hipMemcpyDeviceToDevice, g_stream);
+                if (e != hipSuccess) { sphip_destroy(net); return fail_hip("sphip_clone copy", e); }
+                t.wide_shift = s.wide_shift;
+                t.wide16_valid = true;
+            }
         }
     }
     HCHECK(hipStreamSynchronize(g_stream));
@@ -1582,7 +1649,7 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
         if (fresh[l - 1]) launch_codes16(net->prec, net->W[l - 1].base, codes[l - 1], net->W[l - 1].count);
     // the integer GEMV's quantise launch is never skipped here (that shortcut belongs to the layer timer)
     net->aq_valid_layer = 0;
-    return enqueue_forward(net, wk, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0);
+    return enqueue_forward(net, wk, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS), 0);
 }
 
 int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
@@ -1648,7 +1715,7 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
         HCHECK(hipMemcpyAsync(d_t, targets, out_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
         d_x = net->stage_x;
     }
-    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV), 0)) return 1;
+    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS), 0)) return 1;
     EvalArgs a{d_y, on_dev ? targets : d_t, d_loss, d_pred, d_hit, n, width, loss_func,
                net->act[net->layers - 2] == A_SIGMOID ? 1 : 0};
     sp_eval_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(a);

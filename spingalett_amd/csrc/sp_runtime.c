@@ -74,6 +74,19 @@ SpingalettDequantMode spingalett_get_dequant_mode(void)
     return (SpingalettDequantMode)atomic_load(&g_dequant);
 }
 
+static _Atomic int g_bf16_act = SPINGALETT_BF16_ACTIVATIONS_FP16;
+
+void spingalett_set_bf16_activations(SpingalettBf16Activations mode)
+{
+    if (mode == SPINGALETT_BF16_ACTIVATIONS_BF16 || mode == SPINGALETT_BF16_ACTIVATIONS_FP16)
+        atomic_store(&g_bf16_act, (int)mode);
+}
+
+SpingalettBf16Activations spingalett_get_bf16_activations(void)
+{
+    return (SpingalettBf16Activations)atomic_load(&g_bf16_act);
+}
+
 /* Settings.c:82-110 maps a mode the build lacks to the one it has, with a
  * warning.  This build has exactly one back-end. */
 ComputeMode sp_resolve_compute_mode(void)

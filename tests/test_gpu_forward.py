@@ -286,9 +286,9 @@ def test_scaled_configs(S, O, fmt, topo, acts, n):
 
 _C4S = ([1024] * 9, ["leaky_relu", "foo52"] * 4)             # configuration 4 scaled to 1024-wide layers
 _C5S = ([512, 1024, 1024, 1024, 1024], ["sigmoid", "relu", "relu", "tanh"])
-_BF16_ACT = ("BF16 weights run the BF16 matrix cores with BF16 activations (8 significant bits): measured 99.0-99.3 % "
-             "on 1000 classes, 99.6-99.96 % on 10 classes at 8192 samples")
-_FP16_1000 = ("FP16 activations (11 significant bits) on random 1000-class heads: measured 99.84-99.94 % at 8192 "
+_BF16_ACT = ("the optional setting that runs BF16 weights on the BF16 matrix cores with BF16 activations (8 significant "
+             "bits): measured 99.0-99.3 % on 1000 classes, 99.6-99.96 % on 10 classes at 8192 samples")
+_FP16_1000 = ("FP16 activations (11 significant bits) on random 1000-class heads: measured 99.82-99.94 % at 8192 "
               "samples; the top-2 gap of 1000 random logits is too often below the rounding noise of any 16-bit type")
 
 
@@ -301,16 +301,19 @@ def _xf(reason):
     ("f16", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
     ("i4", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
     ("i2", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
-    pytest.param("bf16", [784, 512, 1000], ["relu", "relu"], 10, "u01", marks=_xf(_BF16_ACT)),
-    ("f16", *_C4S, 10, "n01"), ("i8", *_C4S, 10, "n01"),
-    pytest.param("bf16", *_C4S, 10, "n01", marks=_xf(_BF16_ACT)),
-    pytest.param("bf16", *_C4S, 1000, "n01", marks=_xf(_BF16_ACT)),         # configuration 4's own format and head
+    ("bf16", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
+    ("f16", *_C4S, 10, "n01"), ("i8", *_C4S, 10, "n01"), ("bf16", *_C4S, 10, "n01"),
+    pytest.param("bf16", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),        # configuration 4's own format and head
     pytest.param("f16", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),
     pytest.param("i8", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),
-    ("i2", *_C5S, 10, "u11"), ("i4", *_C5S, 10, "u11"),
+    ("i2", *_C5S, 10, "u11"), ("i4", *_C5S, 10, "u11"), ("bf16", *_C5S, 10, "u11"),
     pytest.param("i2", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),          # configuration 5's own format and head
     pytest.param("i4", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),
-    pytest.param("bf16", *_C5S, 1000, "u11", marks=_xf(_BF16_ACT)),
+    pytest.param("bf16", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),
+    # BF16 weights with spingalett_set_bf16_activations(BF16): BF16 activations on the BF16 matrix cores
+    pytest.param("bf16+bf16act", [784, 512, 1000], ["relu", "relu"], 10, "u01", marks=_xf(_BF16_ACT)),
+    pytest.param("bf16+bf16act", *_C4S, 10, "n01", marks=_xf(_BF16_ACT)),
+    pytest.param("bf16+bf16act", *_C4S, 1000, "n01", marks=_xf(_BF16_ACT)),
 ])
 def test_argmax_agreement_with_the_fp32_reference(S, O, fmt, topo, acts, classes, inp):
     """At least 99.9 % of 8192 samples must have the argmax of the reference's FP32 batch_forward
@@ -318,14 +321,19 @@ def test_argmax_agreement_with_the_fp32_reference(S, O, fmt, topo, acts, classes
     topo = list(topo) + [classes]
     acts = list(acts) + ["softmax"]
     src = make_oracle_net(O, topo, acts, seed=42, bias_std=0.05)
-    _, ref, net = quantized_pair(O, S, src, fmt)
+    bf16act = fmt.endswith("+bf16act")
+    _, ref, net = quantized_pair(O, S, src, fmt.split("+")[0])
     rng = np.random.default_rng(7)
     n = 8192
     X = {"u01": lambda: rng.random((n, topo[0]), dtype=F32), "u11": lambda: rng.random((n, topo[0]), dtype=F32) * 2 - 1,
          "n01": lambda: rng.standard_normal((n, topo[0])).astype(F32)}[inp]()
     fn, _, _ = O.find_sgemm()
     _, want = ref.time_forward_batch(X, 1, fn, 8)
-    got = S.forward_batch(net, X)
+    S.lib().spingalett_set_bf16_activations(1 if bf16act else 0)
+    try:
+        got = S.forward_batch(net, X)
+    finally:
+        S.lib().spingalett_set_bf16_activations(0)
     S.free_network(net)
     assert rel_max_abs(got, want) <= TOL_MFMA
     raw, decided = argmax_agreement(got, want)
@@ -432,6 +440,47 @@ def test_big_tile_gemm_takes_a_partial_k_tile(S, fmt, N, K, n):
     assert _kernel_of(S, net, n) == "sp_gemm16_big"
     assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
     net.destroy()
+
+
+@pytest.mark.parametrize("N,K,n", [
+    (512, 1024, 5), (4096, 2048, 64), (1100, 8192, 200),       # weight-streaming kernel, with and without a K split
+    (16384, 512, 9), (8192, 1024, 8),                          # eight-wave workgroups; K split inside the workgroup
+    (10, 1000, 300), (7, 72, 65),                              # few outputs: activations streamed
+    (768, 1024, 130), (4096, 1000, 4096), (2048, 1000, 2100),  # tiles: K split over the grid, partial K tile
+    (512, 784, 600), (300, 100, 513),                          # single-stage tiles
+])
+def test_bf16_weights_with_fp16_activations(S, N, K, n):
+    """BF16 weights are multiplied on the FP16 matrix cores against an FP16 copy scaled by a power of two, made at
+    upload; SPHIP_BF16_ACTIVATIONS selects the BF16 matrix cores.  Same kernels as FP16 weights (asserted by name
+    against an FP16 net of the same shape), outputs compared with FP64 on the decoded BF16 arrays at the FP16 bound of
+    the other tests; weights spread over 40 binary orders of magnitude in one array, a re-upload, a clone, and the
+    vector path (which has no such copy to use) ride along."""
+    net, W, b = _decoded_layer(S, "bf16", N, K, seed=N + 7 * K + n)
+    ref16, _, _ = _decoded_layer(S, "f16", N, K, seed=1)
+    X = np.random.default_rng(n).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert _kernel_of(S, net, n) == _kernel_of(S, ref16, n)
+    assert rel_max_abs(got, want) <= 1e-3
+    plain = net.forward(X, S.SPHIP_BF16_ACTIVATIONS)           # BF16 activations: the looser bound, and not the same bits
+    assert rel_max_abs(plain, want) <= 4e-3
+    assert not np.array_equal(plain, got)
+    twin = net.clone()
+    assert np.array_equal(twin.forward(X), got)
+    twin.destroy()
+    # a second array: magnitudes from 2^-30 to 2^10 of the largest; what leaves FP16's range is 2^-29 of it and smaller
+    rng = np.random.default_rng(K)
+    w = (rng.standard_normal(N * K) * np.exp2(rng.integers(-30, 11, size=N * K))).astype(F32)
+    codes = (w.view(np.uint32) >> 16).astype(np.uint16)
+    net.upload(0, 0, codes)
+    W2 = (codes.astype(np.uint32) << 16).view(F32).astype(np.float64).reshape(N, K)
+    pre = X.astype(np.float64) @ W2.T + b
+    want2 = np.where(pre > 0, pre, 0.01 * pre)
+    assert rel_max_abs(net.forward(X), want2) <= 1e-3
+    small = net.forward(X[:3])                                 # vector path: FP32 arithmetic on the BF16 array itself
+    assert rel_max_abs(small, want2[:3]) <= 1e-4
+    net.destroy(); ref16.destroy()
 
 
 def _kernel_of(S, net, n, flags=0):
@@ -591,10 +640,10 @@ def test_nonfinite_inputs_through_a_softmax_net(S, O, fmt, n):
 
 
 def test_fp16_activation_range_saturates(S, O):
-    """Matrix-core paths of FP16 and integer weights carry FP16 activations between layers: a finite hidden
-    activation beyond +-65504 becomes +-65504 (documented deviation: the reference keeps FP32 activations,
-    Training.c:327-343), so the outputs equal the oracle's on activations clamped to that range; BF16 weights
-    (BF16 activations, FP32's range) and the vector path at up to four samples do not saturate."""
+    """Matrix-core paths carry FP16 activations between layers: a finite hidden activation beyond +-65504 becomes
+    +-65504 (documented deviation: the reference keeps FP32 activations, Training.c:327-343), so the outputs equal
+    the oracle's on activations clamped to that range; BF16 weights with BF16 activations selected (FP32's range) and
+    the vector path at up to four samples do not saturate."""
     src = make_oracle_net(O, [64, 96, 8], ["none", "none"], seed=93, bias_std=0.0)
     src.W(0)[:] *= 4000.0
     X = np.random.default_rng(94).standard_normal((40, 64)).astype(F32) * 30
@@ -606,7 +655,14 @@ def test_fp16_activation_range_saturates(S, O):
         clamped = np.clip(hidden, -65504, 65504) @ ref.W(1).astype(np.float64).T + ref.b(1)
         got = S.forward_batch(net, X)
         assert np.isfinite(got).all()
-        assert rel_max_abs(got, clamped if fmt == "i8" else full) <= TOL_MFMA
+        assert rel_max_abs(got, clamped) <= TOL_MFMA
+        if fmt == "bf16":
+            S.lib().spingalett_set_bf16_activations(1)
+            try:
+                wide_range = S.forward_batch(net, X)
+            finally:
+                S.lib().spingalett_set_bf16_activations(0)
+            assert rel_max_abs(wide_range, full) <= TOL_MFMA
         assert rel_max_abs(S.forward_batch(net, X[:4]), full[:4]) <= TOL_VEC
         S.free_network(net)
 
@@ -781,10 +837,13 @@ def test_evaluate_batch_argument_checks(S, O):
     S.free_network(net)
 
 
-def test_full_size_gemm_layer_properties(S):
-    """8192 x 8192 BF16 at batch 8192 (one layer of config 4, the tiled GEMM at its benchmark shape):
-    one-hot rows read columns of W exactly, duplicated rows give identical outputs wherever they sit
-    in the batch, and random rows agree with FP64 dot products of the BF16-rounded operands."""
+@pytest.mark.parametrize("activations", ["f16", "bf16"])
+def test_full_size_gemm_layer_properties(S, activations):
+    """8192 x 8192 BF16 at batch 8192 (one layer of config 4, the tiled GEMM at its benchmark shape), with the
+    default FP16 activations and with BF16 activations selected: one-hot rows read columns of W exactly, duplicated
+    rows give identical outputs wherever they sit in the batch, and random rows agree with FP64 dot products of the
+    weights and the inputs rounded to the activation type."""
+    flags = S.SPHIP_BF16_ACTIVATIONS if activations == "bf16" else 0
     K = N = n = 8192
     rng = np.random.default_rng(81)
     w = (rng.standard_normal(N * K, dtype=F32) * F32(0.02))
@@ -800,12 +859,15 @@ def test_full_size_gemm_layer_properties(S):
         X[r, (r * 37 + 5) % K] = 1.0
     X[7000] = X[3]                                                   # duplicates in different tiles
     X[8190] = X[3]
-    Y = net.forward(X)
+    Y = net.forward(X, flags)
     for r in hot:
         assert np.array_equal(Y[r], Wd[:, (r * 37 + 5) % K]), r
     assert np.array_equal(Y[7000], Y[3]) and np.array_equal(Y[8190], Y[3])
     for r in (3, 1234, 8189):
-        xb = ((X[r].view(np.uint32) + 0x7FFF + ((X[r].view(np.uint32) >> 16) & 1)) & 0xFFFF0000).view(F32)   # BF16 RNE
+        if activations == "bf16":
+            xb = ((X[r].view(np.uint32) + 0x7FFF + ((X[r].view(np.uint32) >> 16) & 1)) & 0xFFFF0000).view(F32)   # BF16 RNE
+        else:
+            xb = X[r].astype(np.float16).astype(F32)
         want = Wd.astype(np.float64) @ xb.astype(np.float64)
         assert rel_max_abs(Y[r], want) <= 1e-4, r                    # products exact, FP32 accumulation over 8192 terms
     net.destroy()
