@@ -371,7 +371,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C4", choices=sorted(WORKLOADS) + ["T1"],
                     help="C1..C5: forward configurations; T1: the reference's published training benchmark")
     ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
