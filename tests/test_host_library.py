@@ -385,3 +385,17 @@ int main(void) {
     assert out.stdout.split() == ["3", "24", "9", "160", "1", "8", "2"] + [
         str(v) for v in (C.sizeof(T), T.epochs.offset, T.max_grad_norm.offset, T.autosave_path.offset,
                          T.callback_interval.offset)]
+
+
+def test_bf16_activation_setting_round_trips(S):
+    """spingalett_set_bf16_activations: FP16 activations (0) by default, BF16 (1) on request, anything else ignored."""
+    L = S.lib()
+    assert L.spingalett_get_bf16_activations() == 0
+    try:
+        L.spingalett_set_bf16_activations(1)
+        assert L.spingalett_get_bf16_activations() == 1
+        L.spingalett_set_bf16_activations(7)
+        assert L.spingalett_get_bf16_activations() == 1
+    finally:
+        L.spingalett_set_bf16_activations(0)
+    assert L.spingalett_get_bf16_activations() == 0
