@@ -424,14 +424,16 @@ __device__ __forceinline__ void gemv_i8_specialised(const GemvI8Args &a)
                 *reinterpret_cast<uint32_t *>(dst + 32) = d2;
             };
         };
-        // The activations of a wave's first unit are requested before any weight and have arrived when the stream
-        // waves are let go (barrier "go").
+        // The activations of a wave's first unit are requested before any weight: the stream waves are let go
+        // (barrier "go") as soon as the requests are out, not when the data is in.  A compute unit's memory pipeline
+        // returns data in request order, so the order of the requests is all that has to be right, and the weights
+        // start 0.3-0.45 us earlier per launch (8192 x 8192 INT2 7.86 -> 7.46 us, 16384 x 16384 INT4 29.8 -> 29.4).
         const uint32_t nch0 = cps <= a.nchunks ? cps : a.nchunks;
         if (qid < nch0 * nb) {
             quant_load<FMT>(qr, a.x + (size_t)(qid % nb) * K, K, (qid / nb) * a.kc, a.kc, lane);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __syncthreads();                                      // barrier "go"
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         for (uint32_t s = 0; s < nstages; ++s) {
             const uint32_t ch0 = s * cps, nch = ch0 + cps <= a.nchunks ? cps : a.nchunks - ch0;
             uint8_t *buf = A_lds + (size_t)(s & 1u) * buf_bytes;
@@ -476,7 +478,7 @@ __device__ __forceinline__ void gemv_i8_specialised(const GemvI8Args &a)
             gload16_async(dst[u], wrow + off);
         }
     };
-    __syncthreads();                                              // barrier "go": the quant waves hold their activations
+    __syncthreads();                                              // barrier "go": the quant waves have requested their activations
     u32x4 R[D][G];
 #pragma unroll
     for (int d = 0; d < D; ++d)
