@@ -1418,19 +1418,19 @@ void sphip_destroy(sphip_net *net)
 
 // A BF16 weight array's FP16 copy for the matrix-core path with FP16 activations: the weights times the power of
 // two that brings the array's largest magnitude into [2^14, 2^15).  One small reduction, one wait, one conversion.
-uint32_t *g_absmax_word = nullptr;
-
+// The word the reduction leaves its result in sits behind the copy, in the same allocation.
 int make_wide(DevArray &wa)
 {
-    if (!g_absmax_word) HCHECK(hipMalloc((void **)&g_absmax_word, sizeof(uint32_t)));
-    if (!wa.wide16) HCHECK(hipMalloc((void **)&wa.wide16, wa.count * sizeof(uint16_t)));
+    const size_t copy_bytes = (wa.count * sizeof(uint16_t) + 15u) & ~(size_t)15u;
+    if (!wa.wide16) HCHECK(hipMalloc((void **)&wa.wide16, copy_bytes + 16u));
+    uint32_t *word = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(wa.wide16) + copy_bytes);
     const uint16_t *src = reinterpret_cast<const uint16_t *>(wa.base);
     uint32_t top = 0;
-    HCHECK(hipMemsetAsync(g_absmax_word, 0, sizeof(uint32_t), g_stream));
+    HCHECK(hipMemsetAsync(word, 0, sizeof(uint32_t), g_stream));
     uint64_t blocks = (wa.count + 255) / 256;
     if (blocks > 4096) blocks = 4096;
-    sp_absmax_bf16<<<(uint32_t)blocks, 256, 0, g_stream>>>(src, wa.count, g_absmax_word);
-    HCHECK(hipMemcpyAsync(&top, g_absmax_word, sizeof(uint32_t), hipMemcpyDeviceToHost, g_stream));
+    sp_absmax_bf16<<<(uint32_t)blocks, 256, 0, g_stream>>>(src, wa.count, word);
+    HCHECK(hipMemcpyAsync(&top, word, sizeof(uint32_t), hipMemcpyDeviceToHost, g_stream));
     HCHECK(hipStreamSynchronize(g_stream));
     wa.wide_shift = top ? 14 - ((int)(top >> 7) - 127) : 0;       // largest magnitude = 1.m x 2^(e - 127)
     sp_bf16_to_f16<<<(uint32_t)((wa.count + 255) / 256), 256, 0, g_stream>>>(src, wa.wide16, wa.count, wa.wide_shift);
@@ -1470,7 +1470,7 @@ int sphip_clone(const sphip_net *src, sphip_net **out)
             t.max_val = s.max_val;
             t.uploaded = s.uploaded;
             if (s.wide16_valid) {
-                e = hipMalloc((void **)&t.wide16, s.count * sizeof(uint16_t));
+                e = hipMalloc((void **)&t.wide16, ((s.count * sizeof(uint16_t) + 15u) & ~(size_t)15u) + 16u);
                 if (e == hipSuccess) e = hipMemcpyAsync(t.wide16, s.wide16, s.count * sizeof(uint16_t), hipMemcpyDeviceToDevice, g_stream);
                 if (e != hipSuccess) { sphip_destroy(net); return fail_hip("sphip_clone copy", e); }
                 t.wide_shift = s.wide_shift;
