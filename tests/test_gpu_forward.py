@@ -430,6 +430,8 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096), ("i4", 520, 1056, 300), ("i8", 1100, 2000, 700),
     # ... a single row of 128 x 256 tiles, ragged in M and N, and a K of two tiles and a bit
     ("bf16", 8192, 1000, 100), ("f16", 5000, 1160, 77), ("bf16", 8200, 136, 8200),
+    # output rows that are not whole 16-byte units: one element per lane and store, with and without a K split
+    ("bf16", 4099, 1024, 4096), ("f16", 2001, 1032, 2100), ("i8", 4102, 1040, 3000),
 ])
 def test_big_tile_gemm_takes_a_partial_k_tile(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
