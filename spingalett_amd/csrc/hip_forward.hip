@@ -825,17 +825,28 @@ void launch_gemv(int prec, const Workspace &wk, const LayerArgs &L, const float 
     }
 }
 
-// K splits of the 256 x 256 GEMM when its tiles would leave compute units idle: at least eight K tiles each
-// Rows of a tile of the big GEMM: up to 128 samples a single row of 128 x 256 tiles instead of half-empty 256 x 256
-// ones; for larger batches the smaller tile was measured and is no faster (256 to 2048 samples, 8192-wide layers).
-uint32_t gemm16_tile_rows(uint32_t M)
+// Rows of a tile of the big GEMM.  128 x 256 tiles instead of partly filled or too few 256 x 256 ones: up to 128
+// samples always (a single row of tiles), and for 16-bit weights, which reach LDS by DMA, whenever 256-row tiles
+// would be fewer than 192 (8192 x 8192 BF16 at 256 / 512 / 1024 samples 47.9 / 79.5 / 137 against 53.5 / 82.3 / 150 us,
+// 4096 x 4096 at 1024 samples 50.5 against 54.4, 8192 x 2048 FP16 at 768 samples 37.7 against 64.2 us: twice the
+// tiles, half the K splits or none).  Integer weights pass through registers and are unpacked once per tile: half the
+// rows per unpacked tile cost more than the tiles bring (8192 x 8192 INT2 at 512 samples 93.9 against 81.5 us, INT8
+// at 1024 samples 171 against 162).  With enough 256 x 256 tiles the smaller tile is no faster (8192-wide layers
+// from 1536 samples).
+uint32_t gemm16_tile_rows(int fmt, uint32_t M, uint32_t N)
 {
-    return M <= 128u ? 128u : 256u;
+    if (M <= 128u) return 128u;
+    if (fmt_bits(fmt) != 16) return 256u;
+    // ... and 128-row tiles are at most one per compute unit (more of them run in two rounds, the second mostly
+    // empty: 8192 x 8192 at 1100 samples 242 against 225 us)
+    const uint32_t cols = (N + 255u) / 256u;
+    return ((M + 255u) / 256u) * cols < 192u && ((M + 127u) / 128u) * cols <= 256u ? 128u : 256u;
 }
 
-uint32_t gemm16_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
+// K splits of the tile GEMM when its tiles would leave compute units idle: at least eight K tiles each
+uint32_t gemm16_splits(int fmt, uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 {
-    const uint32_t bm = gemm16_tile_rows(M);
+    const uint32_t bm = gemm16_tile_rows(fmt, M, N);
     const uint32_t tiles = ((M + bm - 1) / bm) * ((N + 255u) / 256u), ktiles = (K + 63u) / 64u;
     *kper = 0;
     if (tiles >= 192u || ktiles < 16u) return 1;
@@ -1040,9 +1051,9 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
     // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
-    const uint32_t bm = gemm16_tile_rows(M);
+    const uint32_t bm = gemm16_tile_rows(FMT, M, L.N);
     const uint32_t big_tiles = ((M + bm - 1) / bm) * ((L.N + 255u) / 256u);
-    const uint32_t splits = gemm16_splits(M, L.N, L.K, &g.kper);
+    const uint32_t splits = gemm16_splits(FMT, M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
     if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
@@ -1051,7 +1062,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         tl_route.name = "sp_gemm16_big";
         if (tl_route.dry) return;
         if (bm == 128u) {
-            // a single row of tiles: 128 rows instead of 256 half-empty ones
+            // 128-row tiles (gemm16_tile_rows)
             constexpr size_t lds = 2 * (128 + 256) * 64 * sizeof(uint16_t);
             auto kern = sp_gemm16_big<FMT, F16T, 2, 4, 2, 2>;
             static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
@@ -1190,7 +1201,7 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n)
             if (tp.use) {
                 if (tp.splits > 1) ws = (uint64_t)tp.splits * tp.NC * tp.R;
             } else {
-                const uint32_t sp = gemm16_splits(n, N, K, &kper);
+                const uint32_t sp = gemm16_splits(net->prec, n, N, K, &kper);
                 if (sp > 1) ws = (uint64_t)sp * n * N;
             }
         }
