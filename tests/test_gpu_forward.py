@@ -286,38 +286,38 @@ def test_scaled_configs(S, O, fmt, topo, acts, n):
 
 _C4S = ([1024] * 9, ["leaky_relu", "foo52"] * 4)             # configuration 4 scaled to 1024-wide layers
 _C5S = ([512, 1024, 1024, 1024, 1024], ["sigmoid", "relu", "relu", "tanh"])
-_BF16_ACT = ("the optional setting that runs BF16 weights on the BF16 matrix cores with BF16 activations (8 significant "
-             "bits): measured 99.0-99.3 % on 1000 classes, 99.6-99.96 % on 10 classes at 8192 samples")
-_FP16_1000 = ("FP16 activations (11 significant bits) on random 1000-class heads: measured 99.82-99.94 % at 8192 "
-              "samples; the top-2 gap of 1000 random logits is too often below the rounding noise of any 16-bit type")
+_C2S = ([784, 512, 1000], ["relu", "relu"])                  # configuration 2
 
-
-def _xf(reason):
-    return pytest.mark.xfail(reason=reason, strict=False)
-
-
-@pytest.mark.parametrize("fmt,topo,acts,classes,inp", [
-    ("i8", [784, 512, 1000], ["relu", "relu"], 10, "u01"),                  # configuration 2
-    ("f16", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
-    ("i4", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
-    ("i2", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
-    ("bf16", [784, 512, 1000], ["relu", "relu"], 10, "u01"),
+# (format, hidden topology, hidden activations, classes, inputs).  "+bf16act": BF16 weights with
+# spingalett_set_bf16_activations(BF16), i.e. BF16 activations on the BF16 matrix cores.
+_ARGMAX_CASES = [
+    ("i8", *_C2S, 10, "u01"), ("f16", *_C2S, 10, "u01"), ("i4", *_C2S, 10, "u01"), ("i2", *_C2S, 10, "u01"),
+    ("bf16", *_C2S, 10, "u01"),
     ("f16", *_C4S, 10, "n01"), ("i8", *_C4S, 10, "n01"), ("bf16", *_C4S, 10, "n01"),
-    pytest.param("bf16", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),        # configuration 4's own format and head
-    pytest.param("f16", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),
-    pytest.param("i8", *_C4S, 1000, "n01", marks=_xf(_FP16_1000)),
+    ("bf16", *_C4S, 1000, "n01"), ("f16", *_C4S, 1000, "n01"), ("i8", *_C4S, 1000, "n01"),   # configuration 4's own head
     ("i2", *_C5S, 10, "u11"), ("i4", *_C5S, 10, "u11"), ("bf16", *_C5S, 10, "u11"),
-    pytest.param("i2", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),          # configuration 5's own format and head
-    pytest.param("i4", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),
-    pytest.param("bf16", *_C5S, 1000, "u11", marks=_xf(_FP16_1000)),
-    # BF16 weights with spingalett_set_bf16_activations(BF16): BF16 activations on the BF16 matrix cores
-    pytest.param("bf16+bf16act", [784, 512, 1000], ["relu", "relu"], 10, "u01", marks=_xf(_BF16_ACT)),
-    pytest.param("bf16+bf16act", *_C4S, 10, "n01", marks=_xf(_BF16_ACT)),
-    pytest.param("bf16+bf16act", *_C4S, 1000, "n01", marks=_xf(_BF16_ACT)),
-])
-def test_argmax_agreement_with_the_fp32_reference(S, O, fmt, topo, acts, classes, inp):
-    """At least 99.9 % of 8192 samples must have the argmax of the reference's FP32 batch_forward
-    (Training.c:313-345, the oracle's sgemm leg on the same decoded weights), and every decided sample."""
+    ("i2", *_C5S, 1000, "u11"), ("i4", *_C5S, 1000, "u11"), ("bf16", *_C5S, 1000, "u11"),   # configuration 5's own head
+    ("bf16+bf16act", *_C2S, 10, "u01"), ("bf16+bf16act", *_C4S, 10, "n01"), ("bf16+bf16act", *_C4S, 1000, "n01"),
+]
+# Raw argmax agreement known to miss 99.9 %, with the floor each case must still hold (a regression guard: the miss
+# is a property of 16-bit activations, not a licence for anything worse).  Measured at 8192 samples: FP16
+# activations (11 significant bits) on random 1000-class heads 99.82-99.94 %; BF16 activations (8 bits) 99.0-99.3 %
+# on 1000 classes and 99.6-99.96 % on 10.
+_ARGMAX_KNOWN_MISS = {
+    ("bf16", 1024, 1000): 0.9975, ("f16", 1024, 1000): 0.9975,
+    ("i8", 1024, 1000): 0.9975,            # 99.94 % measured: passes today, five misses from the bar
+    ("i2", 512, 1000): 0.9975, ("i4", 512, 1000): 0.9975, ("bf16", 512, 1000): 0.9975,
+    ("bf16+bf16act", 784, 10): 0.994, ("bf16+bf16act", 1024, 10): 0.997, ("bf16+bf16act", 1024, 1000): 0.988,
+}
+_argmax_cache = {}
+
+
+def _argmax_case(S, O, fmt, topo, acts, classes, inp, flags_setter=None, tag=""):
+    """GPU outputs and the FP32 reference's (Training.c:313-345: the oracle's sgemm leg on the same decoded weights)
+    for 8192 samples of one case; computed once per case and setting."""
+    key = (fmt, tuple(topo), classes, inp, tag)
+    if key in _argmax_cache:
+        return _argmax_cache[key]
     topo = list(topo) + [classes]
     acts = list(acts) + ["softmax"]
     src = make_oracle_net(O, topo, acts, seed=42, bias_std=0.05)
@@ -330,15 +330,45 @@ def test_argmax_agreement_with_the_fp32_reference(S, O, fmt, topo, acts, classes
     fn, _, _ = O.find_sgemm()
     _, want = ref.time_forward_batch(X, 1, fn, 8)
     S.lib().spingalett_set_bf16_activations(1 if bf16act else 0)
+    if flags_setter:
+        flags_setter(True)
     try:
         got = S.forward_batch(net, X)
     finally:
         S.lib().spingalett_set_bf16_activations(0)
+        if flags_setter:
+            flags_setter(False)
     S.free_network(net)
+    _argmax_cache[key] = (got, want)
+    return got, want
+
+
+@pytest.mark.parametrize("fmt,topo,acts,classes,inp", _ARGMAX_CASES)
+def test_matrix_core_outputs_within_tolerance_of_the_fp32_reference(S, O, fmt, topo, acts, classes, inp):
+    """Every case of the argmax test below, the known misses included: outputs within 2e-2 (relative max-abs) of the
+    reference's FP32 batch_forward, and every decided sample (reference top-2 gap above twice the largest deviation)
+    has the reference's argmax.  No case is excused from these two."""
+    got, want = _argmax_case(S, O, fmt, topo, acts, classes, inp)
     assert rel_max_abs(got, want) <= TOL_MFMA
-    raw, decided = argmax_agreement(got, want)
+    _, decided = argmax_agreement(got, want)
     assert decided == 1.0, decided
-    assert raw >= 0.999, raw
+
+
+@pytest.mark.parametrize("fmt,topo,acts,classes,inp", _ARGMAX_CASES)
+def test_argmax_agreement_with_the_fp32_reference(S, O, fmt, topo, acts, classes, inp):
+    """At least 99.9 % of 8192 samples must have the argmax of the reference's FP32 batch_forward.  The cases known to
+    miss it must hold their floor and are then reported as expected failures with the measured figure; only this one
+    comparison is excused for them."""
+    got, want = _argmax_case(S, O, fmt, topo, acts, classes, inp)
+    raw, _ = argmax_agreement(got, want)
+    floor = _ARGMAX_KNOWN_MISS.get((fmt, topo[0], classes))
+    if floor is None:
+        assert raw >= 0.999, raw
+        return
+    assert raw >= floor, raw
+    if raw < 0.999:
+        pytest.xfail(f"raw argmax agreement {raw:.4%} of 8192 samples (needs more significant bits than a 16-bit "
+                     "activation type has)")
 
 
 def _decoded_layer(S, fmt, N, K, seed):
@@ -720,6 +750,61 @@ def test_batch_permutation_and_row_independence(S, O):
     b = S.forward_batch(net, X[perm])
     assert np.array_equal(a[perm], b)
     S.free_network(net)
+
+
+@pytest.mark.parametrize("fmt,topo,acts,n", [
+    # 16-bit activation buffers of more than 128 MiB: the batch runs as equal blocks of rows, all layers per block
+    ("i2", [64, 8192, 1000], ["relu", "softmax"], 9000),          # 3 blocks of 3072 rows (the last one smaller: 2856)
+    ("bf16", [32, 16384, 24], ["tanh", "none"], 4500),            # 3 blocks of 1536 rows, ragged remainder 1428
+])
+def test_large_batches_run_in_blocks_of_rows(S, fmt, topo, acts, n):
+    """A batch cut into blocks of rows gives the whole batch's outputs (rows are independent; Training.c:313-345 has
+    one sgemm over all rows): against SPHIP_WHOLE_BATCH within FP32 rounding (the K splits of a block may differ from
+    those of the whole batch), and bit for bit against the blocks run as separate calls."""
+    act = {"relu": S.ACT_RELU, "softmax": S.ACT_SOFTMAX, "tanh": S.ACT_TANH, "none": S.ACT_NONE}
+    prec = {"i2": S.PRECISION_INT2, "bf16": S.PRECISION_BFLOAT16}[fmt]
+    rng = np.random.default_rng(n)
+    net = S.DeviceNet(topo, [act[a] for a in acts], prec)
+    for l in range(len(topo) - 1):
+        K, N = topo[l], topo[l + 1]
+        if fmt == "bf16":
+            w = (rng.standard_normal(N * K) * np.sqrt(1.0 / K)).astype(F32)
+            net.upload(l, 0, (w.view(np.uint32) >> 16).astype(np.uint16))
+            net.upload(l, 1, ((rng.standard_normal(N) * 0.1).astype(F32).view(np.uint32) >> 16).astype(np.uint16))
+        else:
+            net.upload(l, 0, rng.integers(0, 256, size=(N * K * 2 + 7) // 8, dtype=np.uint8), 0.5 / np.sqrt(K))
+            net.upload(l, 1, rng.integers(0, 256, size=(N * 2 + 7) // 8, dtype=np.uint8), 0.1)
+    X = rng.standard_normal((n, topo[0])).astype(F32)
+    whole = net.forward(X, S.SPHIP_WHOLE_BATCH)
+    blocks = net.forward(X)
+    assert np.isfinite(whole).all()
+    assert rel_max_abs(blocks, whole) <= 1e-5
+    per_row = 2 * max(topo)
+    rows = (64 << 20) // per_row // 256 * 256
+    nb = -(-n // rows)
+    rows = -(-(-(-n // nb)) // 256) * 256
+    assert rows < n
+    parts = np.concatenate([net.forward(X[r0:r0 + rows], S.SPHIP_WHOLE_BATCH) for r0 in range(0, n, rows)])
+    assert np.array_equal(blocks.view(np.uint32), parts.view(np.uint32))
+    net.destroy()
+
+
+def test_integer_gemv_with_a_very_long_row_falls_back_to_the_vector_kernel(S):
+    """A K so long that the self-quantising integer GEMV's two digit-plane buffers plus its scale records exceed the
+    LDS of a compute unit (2 M columns at four samples: 64 KB of scale records next to two 48 KB plane buffers): the layer must route to the vector kernel, not fail at
+    launch; and it must still compute the product."""
+    K, N, n = 1 << 21, 16, 4
+    rng = np.random.default_rng(5)
+    net = S.DeviceNet([K, N], [S.ACT_NONE], S.PRECISION_INT8)
+    codes = rng.integers(-127, 128, size=N * K, dtype=np.int8)
+    net.upload(0, 0, codes.view(np.uint8), 0.25)
+    net.upload(0, 1, np.zeros(N, np.uint8), 0.0)
+    assert _kernel_of(S, net, n) == "sp_gemv"
+    assert _kernel_of(S, net, 1) in ("sp_gemv", "sp_gemv_i8mfma")
+    X = rng.standard_normal((n, K)).astype(F32)
+    want = X.astype(np.float64) @ (codes.reshape(N, K).astype(np.float64) * (0.25 / 127.0)).T
+    assert rel_max_abs(net.forward(X), want) <= TOL_VEC
+    net.destroy()
 
 
 def test_device_resident_entry_and_argument_checks(S, O):
