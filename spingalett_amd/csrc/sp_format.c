@@ -251,7 +251,7 @@ static NeuralNetwork *load_from_blob(uint8_t *blob, size_t bytes, const char *la
     if (has_opt && !take(&c, &time_step, 8)) FAIL("load: failed to read time step");
     if (!take(&c, &prec, 1) || prec >= PRECISION_COUNT) FAIL("load: invalid precision type");
     if (c.left / 4u < layers) FAIL("load: failed to read topology");
-    const uint32_t *topo_raw = (const uint32_t *)(const void *)c.p;   /* may be unaligned: copy below */
+    const uint8_t *topo_raw = c.p;                    /* unaligned in the file: copied, never read in place */
     uint32_t *topology = (uint32_t *)malloc((size_t)layers * 4u);
     uint8_t *acts = (uint8_t *)malloc(layers - 1);
     if (!topology || !acts) {
