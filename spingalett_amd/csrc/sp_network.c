@@ -8,6 +8,7 @@
 
 #include <math.h>
 #include <pthread.h>
+#include <stdatomic.h>
 #include <stdlib.h>
 #include <string.h>
 #include <time.h>
@@ -117,6 +118,11 @@ void print_parameters(NeuralNetwork *net)
 static pthread_mutex_t g_live_mu = PTHREAD_MUTEX_INITIALIZER;
 static sp_net **g_live = NULL;
 static size_t g_live_n = 0, g_live_cap = 0;
+/* Changes whenever the table does.  A thread remembers the last net it looked up together with this count, so the
+   single-sample latency path neither takes the lock nor scans the table while no net is created or freed. */
+static _Atomic uint64_t g_live_gen = 1;
+static _Thread_local const void *tl_owned_ptr = NULL;
+static _Thread_local uint64_t tl_owned_gen = 0;
 
 static bool live_add(sp_net *sn)
 {
@@ -128,6 +134,7 @@ static bool live_add(sp_net *sn)
         if (t) { g_live = t; g_live_cap = cap; } else ok = false;
     }
     if (ok) g_live[g_live_n++] = sn;
+    atomic_fetch_add(&g_live_gen, 1);
     pthread_mutex_unlock(&g_live_mu);
     return ok;
 }
@@ -137,6 +144,7 @@ static void live_remove(sp_net *sn)
     pthread_mutex_lock(&g_live_mu);
     for (size_t i = 0; i < g_live_n; ++i)
         if (g_live[i] == sn) { g_live[i] = g_live[--g_live_n]; break; }
+    atomic_fetch_add(&g_live_gen, 1);
     pthread_mutex_unlock(&g_live_mu);
 }
 
@@ -144,11 +152,17 @@ sp_net *sp_owned(const NeuralNetwork *net)
 {
     sp_net *found = NULL;
     if (!net) return NULL;
+    if ((const void *)net == tl_owned_ptr && atomic_load(&g_live_gen) == tl_owned_gen)
+        return (sp_net *)(uintptr_t)net;              /* looked up before, and the table has not changed since */
     pthread_mutex_lock(&g_live_mu);
     for (size_t i = 0; i < g_live_n; ++i)
         if ((const void *)g_live[i] == (const void *)net) { found = g_live[i]; break; }
+    const uint64_t gen = atomic_load(&g_live_gen);
     pthread_mutex_unlock(&g_live_mu);
-    return (found && found->magic == SP_NET_MAGIC) ? found : NULL;
+    if (!found || found->magic != SP_NET_MAGIC) return NULL;
+    tl_owned_ptr = net;
+    tl_owned_gen = gen;
+    return found;
 }
 
 /* ---- new_spingalett (Network.c:34-45) ---- */
