@@ -52,7 +52,9 @@ WORKLOADS = {
     "C4": dict(topo=[8192] * 9 + [1000], acts=["leaky", "foo52"] * 4 + ["softmax"], init=["he"] * 9,
                prec=S.PRECISION_BFLOAT16, inputs="n01", batches=[8192]),
     "C5": dict(topo=[2048, 8192, 8192, 8192, 8192, 1000], acts=["sigmoid", "relu", "relu", "tanh", "softmax"],
-               init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1, 8, 64, 512, 4096, 65536]),
+               init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1 << i for i in range(17)],
+               # the batches whose dominant layer is also timed on its own (a roofline entry per row)
+               roofline_batches=[1, 8, 64, 512, 4096, 65536]),
 }
 
 
@@ -236,7 +238,43 @@ def cpu_baseline(path, cfg, n_sample, budget_s=12.0):
     iters = int(max(1, min(200, budget_s / max(sec, 1e-6))))
     sec, _ = net.time_forward_batch(X, iters, sgemm, cores)
     return dict(value=n_sample / sec, unit="samples/s", cores=cores, kind="port",
-                sample=f"{n_sample} samples x {iters} iterations of the same net on host cores, {desc}")
+                sample=f"{n_sample} samples x {iters} iterations of the same net, sgemm NT + bias + activation, {blas_short(desc)}")
+
+
+def blas_short(desc: str) -> str:
+    """'libscipy_openblas-....so (OpenBLAS 0.3.28 DYNAMIC_ARCH ...)' -> 'OpenBLAS 0.3.28 (libscipy_openblas)'"""
+    import re
+    m = re.search(r"OpenBLAS ([0-9.]+)", desc)
+    lib = desc.split("-")[0].split(".so")[0].split(" ")[0]
+    return f"OpenBLAS {m.group(1)} ({lib})" if m else desc[:60]
+
+
+def cpu_baseline_single(path, cfg, budget_s=2.0):
+    """The public single-sample forward's call sequence on the host (Network.c:218-247: bias copy, cblas_sgemv or an
+    OpenMP loop over rows of AVX-style dot products, activation), timed on one seeded input."""
+    import oracle as O
+    with open(path, "rb") as f:
+        blob = f.read()
+    net = O.Net.parse(blob)
+    del blob
+    _, desc, set_threads = O.find_sgemm()
+    sgemv = O.find_sgemv()
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    if set_threads is not None:
+        set_threads(cores)
+    x = make_inputs(cfg["inputs"], 1, cfg["topo"][0], seed=11)[0]
+    out = {}
+    for leg, fn in (("sgemv", sgemv), ("openmp_dot", None)):
+        if leg == "sgemv" and fn is None:
+            continue
+        sec, _ = net.time_forward_single(x, 1, fn, cores)
+        iters = int(max(1, min(500, budget_s / 2 / max(sec, 1e-6))))
+        sec, _ = net.time_forward_single(x, iters, fn, cores)
+        out[leg + "_us"] = sec * 1e6
+    best = min(out.values())
+    return dict(value=1e6 / best, unit="samples/s", cores=cores, kind="port", **out,
+                sample=f"one sample, the public forward's call sequence, {blas_short(desc)} sgemv and OpenMP dot rows")
 
 
 def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0.0):
@@ -257,7 +295,8 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
                    hbm_frac=algorithmic_bytes(topo, prec, n) / (ms_ev * 1e-3) / HBM_PEAK,
                    mfma_frac=fl / (ms_ev * 1e-3) / (FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK),
                    copies=len(copies), finite=bool(np.isfinite(y).all()))
-        row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
+        if n in cfg.get("roofline_batches", batches):
+            row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
         if prec == S.PRECISION_BFLOAT16 and n >= 5:
             # the same workload with BF16 activations on the BF16 matrix cores (SPHIP_BF16_ACTIVATIONS /
             # spingalett_set_bf16_activations): the faster, less accurate setting; the figures above are the default's
@@ -288,7 +327,50 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
             cpu = dict(error=str(e))
         for row in rows:
             row["cpu_baseline"] = cpu
+            if row["batch"] == 1:
+                try:
+                    row["cpu_baseline_b1"] = cpu_baseline_single(path, cfg, cpu_budget_s)
+                except Exception as e:
+                    row["cpu_baseline_b1"] = dict(error=str(e))
     return dict(net=net, path=path, copies=copies, clones=clones, rows=rows, build_s=build_s)
+
+
+def monotone_below(rows, limit=4096):
+    """True when samples/s never drops as the batch doubles, up to `limit` samples (rows of one workload)."""
+    rs = sorted((r for r in rows if r["batch"] <= limit), key=lambda r: r["batch"])
+    return all(b["samples_per_s"] >= a["samples_per_s"] for a, b in zip(rs, rs[1:]))
+
+
+def sig(x, digits=4):
+    """Floats rounded to `digits` significant digits, recursively (the line must stay short enough to be kept whole)."""
+    if isinstance(x, float):
+        return float(f"{x:.{digits}g}") if np.isfinite(x) else None
+    if isinstance(x, dict):
+        return {k: sig(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [sig(v, digits) for v in x]
+    return x
+
+
+def compact_row(row):
+    """One workload row with short keys: w workload, b batch, ms per step (wall), sps samples/s, hbm / mfma whole-net
+    fractions of the peaks, dom the dominant layer's kernel on its own (k kernel, l layer, frac of its bound's peak,
+    ms average launch, traffic HBM-side bytes per launch), fwd_us the public forward() host to host."""
+    if "error" in row:
+        return row
+    out = dict(w=row["workload"], b=row["batch"], ms=row["ms_per_step"], sps=row["samples_per_s"],
+               hbm=row["hbm_frac"], mfma=row["mfma_frac"])
+    if not row["finite"]:
+        out["finite"] = False
+    rl = row.get("roofline")
+    if rl:
+        out["dom"] = dict(k=rl["kernel"], l=rl["layer"], bound=rl["bound"], frac=rl["frac"], ms=rl["avg_ms"],
+                          traffic=rl["traffic"])
+    if "public_forward_us" in row:
+        out["fwd_us"] = row["public_forward_us"]
+    if "cpu_baseline_b1" in row:
+        out["cpu_b1"] = row["cpu_baseline_b1"]
+    return out
 
 
 # The reference's own published benchmark (Examples/Benchmark.c:14-98, README.md:48-59): train() on
@@ -419,14 +501,18 @@ def main():
         cpu = cpu_baseline(head["path"], cfg, sample)
     release(head)
 
-    extra = []
+    extra, cpu_extra, monotone = [], {}, {}
     if not args.no_extra:
         for name in ("C2", "C3", "C5", "C1"):
             if name == args.workload:
                 continue
             try:
                 w = run_workload(name, WORKLOADS[name]["batches"], 50, 3, cpu_budget_s=0.0 if args.no_cpu else 2.0)
-                extra += w["rows"]
+                extra += [compact_row(r) for r in w["rows"]]
+                if w["rows"] and "cpu_baseline" in w["rows"][0]:
+                    cpu_extra[name] = w["rows"][0]["cpu_baseline"]
+                if len(w["rows"]) > 3:
+                    monotone[name] = monotone_below(w["rows"])
                 release(w)
             except Exception as e:  # keep the headline even if an extra configuration fails
                 extra.append(dict(workload=name, error=str(e)))
@@ -452,10 +538,14 @@ def main():
         "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
         "bf16_activations": row.get("bf16_activations"),
         "cpu_baseline": cpu,
+        # the other configurations, one short row per batch (keys: compact_row), their CPU legs once per configuration,
+        # and whether samples/s is monotone in the batch up to 4096 samples (the GEMV -> GEMM crossover)
         "workloads": extra,
+        "cpu_baselines": cpu_extra,
+        "monotone_to_4096": monotone,
         "training": training,
     }
-    print(json.dumps(out))
+    print(json.dumps(sig(out), separators=(",", ":")))
     return 0
 
 

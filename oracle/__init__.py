@@ -84,6 +84,8 @@ def lib():
     L.orc_forward_batch_f64.argtypes = [P(_Net), C.c_void_p, C.c_uint32, C.c_void_p]
     L.orc_time_forward_batch.restype = C.c_double
     L.orc_time_forward_batch.argtypes = [P(_Net), C.c_void_p, C.c_uint32, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+    L.orc_time_forward_single.restype = C.c_double
+    L.orc_time_forward_single.argtypes = [P(_Net), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
     L.orc_sample_loss.restype = C.c_float
     L.orc_sample_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_int, C.c_int]
     L.orc_batch_loss.restype = C.c_float
@@ -218,6 +220,15 @@ class Net:
         sec = lib().orc_time_forward_batch(self._h, _ptr(X), X.shape[0], _ptr(out), iters, fn, threads)
         return sec, out
 
+    def time_forward_single(self, x: np.ndarray, iters: int, sgemv=None, threads: int = 0):
+        """(seconds per call, outputs) of the public single-sample forward's call sequence (Network.c:218-247) with a
+        cblas_sgemv found at run time, or with sgemv=None its OpenMP loop over rows of dot products."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(self.topology[0])
+        out = np.empty(self.topology[-1], dtype=np.float32)
+        fn = C.cast(sgemv, C.c_void_p) if sgemv is not None else None
+        sec = lib().orc_time_forward_single(self._h, _ptr(x), _ptr(out), iters, fn, threads)
+        return sec, out
+
     def batch_gradients(self, X: np.ndarray, T: np.ndarray, grad_scale: float | None = None):
         """(gW, gB, outputs) of one batch: flat arrays laid out like weights / biases."""
         X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, self.topology[0])
@@ -300,6 +311,15 @@ def argmax_rows(outputs: np.ndarray) -> np.ndarray:
 # --------------------------------------------------------------------------
 # BLAS discovery for the CPU-baseline leg
 # --------------------------------------------------------------------------
+def find_sgemv():
+    """cblas_sgemv of the same library find_sgemm() uses (None if there is none)."""
+    fn, _, _ = find_sgemm()
+    return _sgemv_of.get(id(fn)) if fn is not None else None
+
+
+_sgemv_of = {}
+
+
 def find_sgemm():
     """Locate a cblas_sgemm at run time.
 
@@ -320,6 +340,8 @@ def find_sgemm():
             fn = getattr(h, prefix + "cblas_sgemm")
         except (OSError, AttributeError):
             continue
+        if hasattr(h, prefix + "cblas_sgemv"):
+            _sgemv_of[id(fn)] = getattr(h, prefix + "cblas_sgemv")
         setter = None
         for name in (prefix + "openblas_set_num_threads", "openblas_set_num_threads"):
             if hasattr(h, name):

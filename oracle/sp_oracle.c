@@ -757,3 +757,65 @@ double orc_time_forward_batch(const orc_net *n, const float *X, uint32_t N, floa
     free(a); free(b);
     return ((double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec)) / (iters > 0 ? iters : 1);
 }
+
+/* CPU-baseline leg of the public single-sample forward (Network.c:218-247): per layer y = bias (memcpy, :227), then
+ * either cblas_sgemv NoTrans with alpha = beta = 1 (:229-236) or an OpenMP loop over the output rows, each a dot
+ * product with four 8-wide accumulators over 32-float blocks and a scalar tail (:238-245 with SIMD.c:190-240), then
+ * the activation (:247). */
+typedef void (*sgemv_t)(int order, int trans, int m, int n, float alpha, const float *a, int lda, const float *x,
+                        int incx, float beta, float *y, int incy);
+
+static float dot_rows(const float *a, const float *b, uint32_t n)
+{
+    float p[4][8] = {{0}};
+    uint32_t k = 0;
+    for (; k + 32 <= n; k += 32)
+        for (int u = 0; u < 4; ++u)
+            for (int v = 0; v < 8; ++v) p[u][v] += a[k + 8 * u + v] * b[k + 8 * u + v];
+    for (; k + 8 <= n; k += 8)
+        for (int v = 0; v < 8; ++v) p[0][v] += a[k + v] * b[k + v];
+    float q[8];
+    for (int v = 0; v < 8; ++v) q[v] = (p[0][v] + p[1][v]) + (p[2][v] + p[3][v]);
+    float acc = ((q[0] + q[4]) + (q[1] + q[5])) + ((q[2] + q[6]) + (q[3] + q[7]));
+    for (; k < n; ++k) acc += a[k] * b[k];
+    return acc;
+}
+
+static void forward_single_impl(const orc_net *n, const float *x, float *out, sgemv_t gemv, float *cur, float *nxt)
+{
+    memcpy(cur, x, 4u * (size_t)n->topology[0]);
+    for (uint32_t l = 1; l < n->layers; ++l) {
+        const uint32_t in = n->topology[l - 1], o = n->topology[l];
+        const float *W = n->weights + n->woff[l - 1], *b = n->biases + n->boff[l - 1];
+        memcpy(nxt, b, 4u * (size_t)o);
+        if (gemv) {
+            gemv(101 /* row major */, 111 /* no transpose */, (int)o, (int)in, 1.0f, W, (int)in, cur, 1, 1.0f, nxt, 1);
+        } else {
+#if defined(_OPENMP)
+#pragma omp parallel for schedule(static)
+#endif
+            for (int64_t j = 0; j < (int64_t)o; ++j) nxt[j] += dot_rows(cur, W + (uint64_t)j * in, in);
+        }
+        orc_apply_activation(nxt, 1, o, n->act[l - 1]);
+        float *t = cur; cur = nxt; nxt = t;
+    }
+    memcpy(out, cur, 4u * (size_t)n->topology[n->layers - 1]);
+}
+
+double orc_time_forward_single(const orc_net *n, const float *x, float *out, int iters, void *sgemv_fn, int threads)
+{
+#if defined(_OPENMP)
+    if (threads > 0) omp_set_num_threads(threads);
+#else
+    (void)threads;
+#endif
+    uint32_t mw = max_width(n);
+    float *a = (float *)malloc(4u * (size_t)mw), *b = (float *)malloc(4u * (size_t)mw);
+    forward_single_impl(n, x, out, (sgemv_t)sgemv_fn, a, b);       /* warm-up */
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (int i = 0; i < iters; ++i) forward_single_impl(n, x, out, (sgemv_t)sgemv_fn, a, b);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    free(a); free(b);
+    return ((double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec)) / (iters > 0 ? iters : 1);
+}

@@ -154,6 +154,9 @@ void orc_apply_gradients(orc_net *net, const orc_opt_args *args, float *gW, floa
  * OpenMP kernel.  Returns seconds per call averaged over `iters`. */
 double orc_time_forward_batch(const orc_net *net, const float *X, uint32_t N,
                               float *out, int iters, void *sgemm_fn, int threads);
+/* The same for the public single-sample forward (Network.c:218-247): bias copy, then cblas_sgemv (sgemv_fn) or,
+ * with NULL, an OpenMP loop over output rows of 4 x 8-lane dot products (SIMD.c:190-240), then the activation. */
+double orc_time_forward_single(const orc_net *net, const float *x, float *out, int iters, void *sgemv_fn, int threads);
 
 #ifdef __cplusplus
 }

@@ -148,3 +148,28 @@ def test_batch_loss_and_argmax(O):
     assert np.array_equal(O.argmax_rows(Y), Y.argmax(1))
     tie = np.array([[1.0, 3.0, 3.0, 2.0], [5.0, 5.0, 5.0, 5.0]], np.float32)
     assert list(O.argmax_rows(tie)) == [1, 0]                      # first maximum
+
+
+def test_single_sample_baseline_leg_computes_the_forward(O):
+    """The CPU-baseline leg of the public forward (bias copy, sgemv or OpenMP rows of 4 x 8-lane dot products,
+    activation: Network.c:218-247, SIMD.c:190-240) is only ever timed; what it computes must still be the forward:
+    both variants against numpy float64 on a ragged net whose widths exercise the 32-, 8- and 1-element steps."""
+    rng = np.random.default_rng(11)
+    topo, acts = [301, 77, 45, 9], ["relu", "tanh", "softmax"]
+    net = O.Net.new(topo, [O.ACT[a] for a in acts], 1)
+    for l in range(3):
+        net.W(l)[:] = (rng.standard_normal(net.W(l).shape) * 0.2).astype(np.float32)
+        net.b(l)[:] = (rng.standard_normal(net.b(l).shape) * 0.1).astype(np.float32)
+    x = rng.standard_normal(topo[0]).astype(np.float32)
+    a = x.astype(np.float64)
+    for l, act in enumerate(acts):
+        z = net.W(l).astype(np.float64) @ a + net.b(l)
+        a = {"relu": lambda z: np.maximum(z, 0), "tanh": np.tanh,
+             "softmax": lambda z: np.exp(z - z.max()) / np.exp(z - z.max()).sum()}[act](z)
+    legs = [None]
+    if O.find_sgemv() is not None:
+        legs.append(O.find_sgemv())
+    for fn in legs:
+        sec, out = net.time_forward_single(x, 2, fn, 2)
+        assert sec > 0
+        assert np.abs(out - a).max() <= 1e-5
