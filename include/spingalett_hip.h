@@ -48,6 +48,11 @@ typedef struct {
  * cores instead: 8 instead of 11 significant bits between layers, a few per cent faster.  Other formats and the
  * vector path ignore it; no counterpart in the reference, whose activations are FP32. */
 #define SPHIP_BF16_ACTIVATIONS 32u
+/* A batch whose 16-bit activation buffers would exceed the memory-side cache (more than 128 MiB per buffer) runs as
+ * equal blocks of rows, all layers per block (at most 64 MiB per buffer, a multiple of 256 rows), so that the layer
+ * boundaries stay in that cache; the workspace is sized for a block.  Rows are independent, the outputs are the whole
+ * batch's.  This flag runs the whole batch layer by layer instead (benchmark comparisons). */
+#define SPHIP_WHOLE_BATCH 64u
 
 SPHIP_API int  sphip_device_count(void);
 SPHIP_API const char *sphip_last_error_string(void);   /* per thread */
@@ -152,6 +157,9 @@ SPHIP_API int  sphip_train_step(sphip_net *net, const float *x, const float *tar
 /* ---- measurement helpers (benchmark harness; not part of the data path) ---- */
 SPHIP_API int  sphip_malloc(void **dptr, size_t bytes);
 SPHIP_API int  sphip_free(void *dptr);
+/* Free and total bytes of the current device's memory (hipMemGetInfo): lets a harness check that a call allocated
+ * nothing. */
+SPHIP_API int  sphip_device_memory(size_t *free_bytes, size_t *total_bytes);
 SPHIP_API int  sphip_memcpy_h2d(void *dst, const void *src, size_t bytes);
 SPHIP_API int  sphip_memcpy_d2h(void *dst, const void *src, size_t bytes);
 /* A second device copy of a net's arrays (so a timing loop can rotate over

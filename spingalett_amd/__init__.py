@@ -39,6 +39,7 @@ AUTOSAVE_OFF, AUTOSAVE_OVERWRITE, AUTOSAVE_NEW_FILES = 0, 1, 2
 
 SPHIP_X_ON_DEVICE, SPHIP_Y_ON_DEVICE, SPHIP_FORCE_GEMM, SPHIP_FORCE_GEMV = 1, 2, 8, 16
 SPHIP_BF16_ACTIVATIONS = 32
+SPHIP_WHOLE_BATCH = 64
 (SPHIP_TRAIN_W, SPHIP_TRAIN_B, SPHIP_TRAIN_MW, SPHIP_TRAIN_VW, SPHIP_TRAIN_MB, SPHIP_TRAIN_VB,
  SPHIP_TRAIN_GW, SPHIP_TRAIN_GB) = range(8)
 
@@ -138,6 +139,7 @@ PUBLIC_SYMBOLS = [
 SPHIP_SYMBOLS = [
     "sphip_device_count", "sphip_last_error_string", "sphip_create", "sphip_destroy", "sphip_upload_array",
     "sphip_forward", "sphip_forward_noalloc", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
+    "sphip_device_memory",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
     "sphip_layer_kernel_name", "sphip_evaluate",
     "sphip_train_begin", "sphip_train_end", "sphip_train_set", "sphip_train_get", "sphip_train_step",
@@ -224,6 +226,7 @@ def lib():
     L.sphip_synchronize.restype = C.c_int
     L.sphip_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]; L.sphip_malloc.restype = C.c_int
     L.sphip_free.argtypes = [C.c_void_p]; L.sphip_free.restype = C.c_int
+    L.sphip_device_memory.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]; L.sphip_device_memory.restype = C.c_int
     L.sphip_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]; L.sphip_memcpy_h2d.restype = C.c_int
     L.sphip_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]; L.sphip_memcpy_d2h.restype = C.c_int
     L.sphip_clone.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]; L.sphip_clone.restype = C.c_int
@@ -425,6 +428,13 @@ def hip_decode(net, l: int, which: int) -> np.ndarray:
 def _check(rc: int, what: str):
     if rc:
         raise SpingalettError(f"{what}: {lib().sphip_last_error_string().decode()}")
+
+
+def device_memory():
+    """(free, total) bytes of the device's memory."""
+    f, t = C.c_size_t(), C.c_size_t()
+    _check(lib().sphip_device_memory(C.byref(f), C.byref(t)), "sphip_device_memory")
+    return f.value, t.value
 
 
 class DeviceBuffer:

@@ -780,6 +780,8 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
         a.stage_blocks = stage;
         if (lds < red_bytes) lds = red_bytes;
         lds += a.meta_bytes;
+        // a K so long that two buffers and the scale records no longer fit: the vector kernel takes the layer
+        if (lds > 156u * 1024u) return false;
         // one quant wave per (scale chunk, sample) of the first stage, at most eight.  (Cutting a chunk into slices so
         // that eight waves quantise a K of fewer chunks, the slices' maxima meeting in LDS, was measured: 0.7-0.9 us
         // slower per layer on 8192-wide INT2 / INT8 layers.)
@@ -1352,6 +1354,49 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
     return 0;
 }
 
+// Rows per pass over a large batch.  The activations between two layers are written once and read once; when the
+// two buffers of a whole batch exceed the memory-side cache (256 MB), every layer boundary goes through HBM.  Running
+// all layers over one block of rows after the other keeps the boundaries in that cache (the weights are re-read per
+// block, from HBM or from the same cache).  Rows are independent (Training.c:313-345 computes them by one sgemm, but
+// no row's result depends on another's), so the outputs are those of the whole batch up to the choice of K splits.
+// Blocks are equal, a multiple of 256 rows, and as large as fits 64 MiB per 16-bit activation buffer.  Batches of up
+// to 128 MiB per buffer stay whole: measured on one box, 8192 samples of the 8192-wide BF16 net 7.72 ms whole against
+// 7.82 ms in two blocks (the weights, 128 MiB per layer, are then read twice) and of the 8192-wide INT2 net 2.75
+// against 2.74 ms; 16384 samples of the latter 5.83 against 5.45 ms, 65536 samples 24.0 against 21.6 ms.
+uint32_t batch_block_rows(const sphip_net *net, uint32_t n, uint32_t flags)
+{
+    if ((flags & SPHIP_WHOLE_BATCH) || pick_regime(net, n, flags) != R_GEMM16) return n;
+    const uint64_t per_row = (uint64_t)net->max_width * 2u;
+    if ((uint64_t)n * per_row <= (128ull << 20)) return n;
+    uint64_t rows = (64ull << 20) / per_row / 256u * 256u;
+    if (rows < 1024u) rows = 1024u;
+    if (rows >= n) return n;
+    const uint64_t blocks = (n + rows - 1) / rows;
+    rows = ((n + blocks - 1) / blocks + 255u) / 256u * 256u;
+    return (uint32_t)rows;
+}
+
+// reserve() for a batch that may run in blocks of rows: the workspace of a full block and of the last, smaller one
+int reserve_batch(sphip_net *net, uint32_t n, uint32_t flags)
+{
+    const uint32_t rows = batch_block_rows(net, n, flags);
+    if (reserve(net, rows, false)) return 1;
+    if (rows < n && n % rows != 0 && reserve(net, n % rows, false)) return 1;
+    return 0;
+}
+
+// enqueue_forward over the blocks of rows of batch_block_rows(); the caller has called reserve_batch()
+int enqueue_forward_batch(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags, uint32_t only_layer)
+{
+    const uint32_t rows = batch_block_rows(net, n, flags);
+    const uint32_t in_w = net->topo[0], out_w = net->topo[net->layers - 1];
+    for (uint32_t r0 = 0; r0 < n; r0 += rows) {
+        const uint32_t m = n - r0 < rows ? n - r0 : rows;
+        if (enqueue_forward(net, net->workspace(), d_x + (size_t)r0 * in_w, m, d_y + (size_t)r0 * out_w, flags, only_layer)) return 1;
+    }
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1573,7 +1618,8 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
 {
     if (!net || !x || !y || n == 0) return fail_msg("sphip_forward: invalid argument");
     if (check_uploaded(net)) return 1;
-    if (reserve(net, n, false)) return 1;
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH);
+    if (reserve_batch(net, n, fwd_flags)) return 1;
     const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * net->topo[net->layers - 1];
     const float *d_x = x;
     float *d_y = y;
@@ -1599,7 +1645,7 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
             d_y = net->stage_y;
         }
     }
-    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags, 0)) return 1;
+    if (enqueue_forward_batch(net, d_x, n, d_y, fwd_flags, 0)) return 1;
     if (!(flags & SPHIP_Y_ON_DEVICE)) {
         if (!y_pinned) HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
         HCHECK(hipStreamSynchronize(g_stream));
@@ -1642,9 +1688,12 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
     wk.split_cap = need.split_floats;
     // an integer layer with few outputs reads an FP16 copy of its codes: the net's own if an earlier call made one,
     // else one made here, in the scratch array, on every call
+    // (only the matrix-core regime reads them: a forced vector forward or one of up to four samples never does)
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS);
+    const bool reads_codes = pick_regime(net, n, fwd_flags) == R_GEMM16;
     bool fresh[kMaxLayers] = {};
     for (uint32_t l = 1; l < net->layers; ++l) {
-        if (!layer_wants_codes16(net, l, n)) continue;
+        if (!reads_codes || !layer_wants_codes16(net, l, n)) continue;
         const DevArray &wa = net->W[l - 1];
         if (wa.codes16_valid) { codes[l - 1] = wa.codes16; continue; }
         codes[l - 1] = reinterpret_cast<uint16_t *>(take(wa.count * sizeof(uint16_t)));
@@ -1660,7 +1709,7 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
         if (fresh[l - 1]) launch_codes16(net->prec, net->W[l - 1].base, codes[l - 1], net->W[l - 1].count);
     // the integer GEMV's quantise launch is never skipped here (that shortcut belongs to the layer timer)
     net->aq_valid_layer = 0;
-    return enqueue_forward(net, wk, d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS), 0);
+    return enqueue_forward(net, wk, d_x, n, d_y, fwd_flags, 0);
 }
 
 int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
@@ -1705,7 +1754,8 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
     if (!net || !x || !targets || n == 0 || (loss_func != 0 && loss_func != 1))
         return fail_msg("sphip_evaluate: invalid argument");
     if (check_uploaded(net)) return 1;
-    if (reserve(net, n, false)) return 1;
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH);
+    if (reserve_batch(net, n, fwd_flags)) return 1;
     const uint32_t width = net->topo[net->layers - 1];
     const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * width;
     const bool on_dev = (flags & SPHIP_X_ON_DEVICE) != 0;
@@ -1726,7 +1776,7 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
         HCHECK(hipMemcpyAsync(d_t, targets, out_cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
         d_x = net->stage_x;
     }
-    if (enqueue_forward(net, net->workspace(), d_x, n, d_y, flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS), 0)) return 1;
+    if (enqueue_forward_batch(net, d_x, n, d_y, fwd_flags, 0)) return 1;
     EvalArgs a{d_y, on_dev ? targets : d_t, d_loss, d_pred, d_hit, n, width, loss_func,
                net->act[net->layers - 2] == A_SIGMOID ? 1 : 0};
     sp_eval_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(a);
@@ -1795,6 +1845,14 @@ int sphip_malloc(void **dptr, size_t bytes)
     return 0;
 }
 
+int sphip_device_memory(size_t *free_bytes, size_t *total_bytes)
+{
+    if (!free_bytes || !total_bytes) return fail_msg("sphip_device_memory: null");
+    if (ensure_stream()) return 1;
+    HCHECK(hipMemGetInfo(free_bytes, total_bytes));
+    return 0;
+}
+
 int sphip_free(void *dptr)
 {
     if (dptr) HCHECK(hipFree(dptr));
@@ -1824,14 +1882,14 @@ static int time_common(sphip_net *const *nets, int count, const float *d_x, uint
     for (int i = 0; i < count; ++i) {
         if (!nets[i]) return fail_msg("sphip_time: null net");
         if (check_uploaded(nets[i])) return 1;
-        if (reserve(nets[i], n, false)) return 1;
+        if (reserve_batch(nets[i], n, flags)) return 1;
     }
     TimingEvents ev;
     if (ev.create()) return 1;
     hipEvent_t e0 = ev.e0, e1 = ev.e1;
     int rc = 0;
     HCHECK(hipEventRecord(e0, g_stream));
-    for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward(nets[it % count], nets[it % count]->workspace(), d_x, n, d_y, flags, only_layer);
+    for (int it = 0; it < iters && !rc; ++it) rc = enqueue_forward_batch(nets[it % count], d_x, n, d_y, flags, only_layer);
     hipError_t e = hipEventRecord(e1, g_stream);
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
@@ -1854,7 +1912,7 @@ int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t
         return fail_msg("sphip_time_layer: invalid argument");
     // inputs and outputs are the nets' own scratch buffers (contents irrelevant for timing)
     for (int i = 0; i < count; ++i) {
-        if (reserve(nets[i], n, false)) return 1;
+        if (reserve_batch(nets[i], n, flags)) return 1;
         if (grow(&nets[i]->stage_y, &nets[i]->stage_y_cap, (uint64_t)n * nets[i]->topo[nets[i]->layers - 1])) return 1;
         if (grow(&nets[i]->stage_x, &nets[i]->stage_x_cap, (uint64_t)n * nets[i]->topo[0])) return 1;
     }

@@ -65,6 +65,14 @@ def test_noalloc_forward_equals_forward(S, fmt, topo, acts, ns, flags):
         want = net.forward(X, flags)
         assert np.isfinite(want).all()
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (fmt, n)
+        # What the entry point exists for: a warmed call takes no device memory.  `fresh` has no buffers of its own,
+        # so an allocation on any route of this case would lower the free figure.
+        free_before, _ = S.device_memory()
+        assert fresh.forward_noalloc(d_x, n, d_y, flags) == 0
+        S.synchronize()
+        free_after, _ = S.device_memory()
+        assert free_after == free_before, (fmt, n, free_before - free_after)
+        assert np.array_equal(d_y.to_numpy(F32, (n, topo[-1])).view(np.uint32), want.view(np.uint32)), (fmt, n)
     net.destroy()
     fresh.destroy()
 
