@@ -53,6 +53,13 @@ typedef struct {
  * boundaries stay in that cache; the workspace is sized for a block.  Rows are independent, the outputs are the whole
  * batch's.  This flag runs the whole batch layer by layer instead (benchmark comparisons). */
 #define SPHIP_WHOLE_BATCH 64u
+/* Split activations on the matrix-core path (5 samples and more; any 16-bit or integer weight format): between the
+ * layers every activation travels as two FP16 numbers, hi = the value rounded to FP16 and lo = (value - hi) 2^11, about
+ * 22 significant bits together (the reference keeps FP32 activations, Training.c:313-345).  Each layer multiplies the
+ * weights with both matrices (twice the matrix-core work) into FP32 partial sums that a second launch adds.  For nets
+ * whose decisions hang on differences below FP16's 11 bits (many-class softmax heads); supersedes
+ * SPHIP_BF16_ACTIVATIONS. */
+#define SPHIP_SPLIT_ACTIVATIONS 128u
 
 SPHIP_API int  sphip_device_count(void);
 SPHIP_API const char *sphip_last_error_string(void);   /* per thread */
@@ -89,7 +96,8 @@ SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *
  * A batch whose workspace exceeds the array is refused with an error that names both sizes (sphip_forward takes it).
  * Nothing in the array needs clearing between calls: every kernel reads only what this call wrote.  All calls on one
  * GPU share the array, so two calls that overlap in time (from different threads) race; nets of more than 64 layers
- * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV / SPHIP_BF16_ACTIVATIONS only. */
+ * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV / SPHIP_BF16_ACTIVATIONS /
+ * SPHIP_SPLIT_ACTIVATIONS only. */
 #define SPHIP_NOALLOC_SCRATCH_BYTES (64u << 20)
 SPHIP_API int  sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags);
 /* The evaluation step that follows batch_forward in the reference's epoch loop, on the device:

@@ -39,7 +39,8 @@ AUTOSAVE_OFF, AUTOSAVE_OVERWRITE, AUTOSAVE_NEW_FILES = 0, 1, 2
 
 SPHIP_X_ON_DEVICE, SPHIP_Y_ON_DEVICE, SPHIP_FORCE_GEMM, SPHIP_FORCE_GEMV = 1, 2, 8, 16
 SPHIP_BF16_ACTIVATIONS = 32
-SPHIP_WHOLE_BATCH = 64
+SPHIP_WHOLE_BATCH, SPHIP_SPLIT_ACTIVATIONS = 64, 128
+NET_ACTIVATIONS_DEFAULT, NET_ACTIVATIONS_BF16, NET_ACTIVATIONS_SPLIT = 0, 1, 2
 (SPHIP_TRAIN_W, SPHIP_TRAIN_B, SPHIP_TRAIN_MW, SPHIP_TRAIN_VW, SPHIP_TRAIN_MB, SPHIP_TRAIN_VB,
  SPHIP_TRAIN_GW, SPHIP_TRAIN_GB) = range(8)
 
@@ -131,7 +132,7 @@ PUBLIC_SYMBOLS = [
     "new_spingalett_struct_arguments", "layer_struct_arguments", "activate", "forward_struct_arguments",
     "save_spingalett_struct_arguments", "load_spingalett", "free_network",
     "spingalett_set_dequant_mode", "spingalett_get_dequant_mode", "spingalett_forward_batch",
-    "spingalett_set_bf16_activations", "spingalett_get_bf16_activations",
+    "spingalett_set_bf16_activations", "spingalett_get_bf16_activations", "spingalett_set_net_activations",
     "spingalett_forward_batch_device", "spingalett_hip_synchronize", "spingalett_hip_invalidate",
     "spingalett_hip_precision", "spingalett_hip_decode", "spingalett_hip_handle", "load_spingalett_memory",
     "spingalett_evaluate_batch", "train_struct_arguments", "derivative", "print_parameters",
@@ -193,6 +194,7 @@ def lib():
     L.spingalett_set_dequant_mode.argtypes = [C.c_int]; L.spingalett_set_dequant_mode.restype = None
     L.spingalett_get_dequant_mode.restype = C.c_int
     L.spingalett_set_bf16_activations.argtypes = [C.c_int]; L.spingalett_set_bf16_activations.restype = None
+    L.spingalett_set_net_activations.argtypes = [NetPtr, C.c_int]; L.spingalett_set_net_activations.restype = C.c_int
     L.spingalett_get_bf16_activations.restype = C.c_int
     L.spingalett_forward_batch.argtypes = [NetPtr, C.c_void_p, C.c_uint32, C.c_void_p]
     L.spingalett_forward_batch.restype = C.c_void_p

@@ -95,9 +95,11 @@ static bool ensure_device(sp_net *sn)
     return true;
 }
 
-/* what spingalett_set_bf16_activations asks of the batched entry points */
-static uint32_t activation_flags(void)
+/* what spingalett_set_net_activations, or else spingalett_set_bf16_activations, asks of the batched entry points */
+static uint32_t activation_flags(const sp_net *sn)
 {
+    if (sn->act_mode == SPINGALETT_NET_ACTIVATIONS_SPLIT) return SPHIP_SPLIT_ACTIVATIONS;
+    if (sn->act_mode == SPINGALETT_NET_ACTIVATIONS_BF16) return SPHIP_BF16_ACTIVATIONS;
     return spingalett_get_bf16_activations() == SPINGALETT_BF16_ACTIVATIONS_BF16 ? SPHIP_BF16_ACTIVATIONS : 0u;
 }
 
@@ -131,6 +133,18 @@ float *sp_hip_forward_single(sp_net *sn, const float *input)
     return out;
 }
 
+int spingalett_set_net_activations(NeuralNetwork *net, SpingalettNetActivations mode)
+{
+    sp_net *sn = checked(net, "set_net_activations");
+    if (!sn) return 1;
+    if ((unsigned)mode > SPINGALETT_NET_ACTIVATIONS_SPLIT) {
+        sp_set_error(SPINGALETT_ERR_INVALID, "set_net_activations: unknown mode");
+        return 1;
+    }
+    sn->act_mode = (int)mode;
+    return 0;
+}
+
 float *spingalett_forward_batch(NeuralNetwork *net, const float *inputs, uint32_t n, float *outputs)
 {
     (void)sp_resolve_compute_mode();
@@ -139,7 +153,7 @@ float *spingalett_forward_batch(NeuralNetwork *net, const float *inputs, uint32_
     if (!sn) return NULL;
     if (n == 0) return outputs;
     if (!ensure_device(sn)) return NULL;
-    if (sphip_forward(sn->dev, inputs, n, outputs, activation_flags())) {
+    if (sphip_forward(sn->dev, inputs, n, outputs, activation_flags(sn))) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: forward_batch");
         return NULL;
     }
@@ -155,7 +169,7 @@ int spingalett_forward_batch_device(NeuralNetwork *net, const float *d_inputs, u
         return 1;
     }
     if (!ensure_device(sn)) return 1;
-    if (sphip_forward(sn->dev, d_inputs, n, d_outputs, SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE | activation_flags())) {
+    if (sphip_forward(sn->dev, d_inputs, n, d_outputs, SPHIP_X_ON_DEVICE | SPHIP_Y_ON_DEVICE | activation_flags(sn))) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: forward_batch_device");
         return 1;
     }
@@ -177,7 +191,7 @@ int spingalett_evaluate_batch(NeuralNetwork *net, const float *inputs, const flo
         return 1;
     }
     if (!ensure_device(sn)) return 1;
-    if (sphip_evaluate(sn->dev, inputs, targets, n, (int)net->loss_func, activation_flags(), total_loss, predictions, correct)) {
+    if (sphip_evaluate(sn->dev, inputs, targets, n, (int)net->loss_func, activation_flags(sn), total_loss, predictions, correct)) {
         report(SPINGALETT_ERR_INVALID, "HIP back-end: evaluate_batch");
         return 1;
     }

@@ -106,6 +106,7 @@ hipStream_t g_stream = nullptr;
 struct RouteState {
     bool dry = false;
     const char *name = "";
+    uint32_t halves = 1;            // 2: split activations (SPHIP_SPLIT_ACTIVATIONS), every layer goes through partial sums
 };
 thread_local RouteState tl_route;
 constexpr uint32_t kGemvStageBytes = 64u * 1024u;   // LDS budget of one stage of the integer GEMV
@@ -355,7 +356,7 @@ __global__ __launch_bounds__(256) void sp_decode(const DecodeParams p)
 // ---------------------------------------------------------------------------
 // softmax over rows (Activation.c:5-21); one wave per row
 // ---------------------------------------------------------------------------
-// out_kind: 0 FP32, 1 BF16, 2 FP16
+// out_kind: 0 FP32, 1 BF16, 2 FP16, 3 split FP16 (hi, and (v - hi) 2^11 rows * width elements further on)
 __global__ __launch_bounds__(256) void sp_softmax_rows(const float *__restrict__ in, void *__restrict__ out,
                                                        int out_kind, uint32_t rows, uint32_t width)
 {
@@ -367,7 +368,14 @@ __global__ __launch_bounds__(256) void sp_softmax_rows(const float *__restrict__
         const size_t o = (size_t)row * width + i;
         if (out_kind == 0) reinterpret_cast<float *>(out)[o] = v;
         else if (out_kind == 1) reinterpret_cast<uint16_t *>(out)[o] = f32_to_bf16_rne(v);
-        else reinterpret_cast<uint16_t *>(out)[o] = f32_to_f16_sat(v);
+        else if (out_kind == 2) reinterpret_cast<uint16_t *>(out)[o] = f32_to_f16_sat(v);
+        else {
+            const uint16_t hi = f32_to_f16_sat(v);
+            _Float16 hh;
+            __builtin_memcpy(&hh, &hi, 2);
+            reinterpret_cast<uint16_t *>(out)[o] = hi;
+            reinterpret_cast<uint16_t *>(out)[(size_t)rows * width + o] = f32_to_f16_sat((v - (float)hh) * 2048.0f);
+        }
     };
     constexpr int R = 16;                       // rows up to 1024 wide stay in registers: one batch of loads
     if (width <= (uint32_t)R * kWave) {
@@ -422,6 +430,21 @@ __global__ __launch_bounds__(256) void sp_cvt16(const float *__restrict__ in, ui
     } else {
         for (; i < n; ++i) out[i] = f32_to_t16<F16T>(in[i]);
     }
+}
+
+// FP32 -> the two FP16 matrices of a split activation: hi = the value rounded to FP16, and (value - hi) 2^11, n
+// elements further on (the difference is exact in FP32; infinities and NaNs live in hi alone)
+__global__ __launch_bounds__(256) void sp_cvt16_split(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    const float v = in[i];
+    const uint16_t hi = f32_to_f16_sat(v);
+    _Float16 hh;
+    __builtin_memcpy(&hh, &hi, 2);
+    const float rest = (v - (float)hh) * 2048.0f;
+    out[i] = hi;
+    out[n + i] = (rest == rest && fabsf(rest) != __builtin_inff()) ? f32_to_f16_sat(rest) : (uint16_t)0;
 }
 
 // largest bit pattern of |w| among the finite BF16 values of an array
@@ -978,7 +1001,7 @@ void launch_thin_inst(const SkinnyArgs &a, const ThinPlan &p)
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
     (void)once;
     const uint32_t gx = p.cblocks > 1 ? (p.row_blocks + 7u) / 8u * 8u * p.cblocks : p.row_blocks;
-    kern<<<dim3(gx, p.splits, 1), 64 * NWV, lds, g_stream>>>(a);
+    kern<<<dim3(gx, p.splits * a.halves, 1), 64 * NWV, lds, g_stream>>>(a);
 }
 
 template <int SFMT, bool F16T, int NCP, int NW>
@@ -989,13 +1012,14 @@ void launch_thin_kw(const SkinnyArgs &a, const ThinPlan &p)
     auto kern = sp_skinny16_kw<SFMT, F16T, NCP, NW>;
     static bool once = ((void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
     (void)once;
-    kern<<<dim3(p.row_blocks, p.splits, 1), 64 * NW, lds, g_stream>>>(a);
+    kern<<<dim3(p.row_blocks, p.splits * a.halves, 1), 64 * NW, lds, g_stream>>>(a);
 }
 
 template <int SFMT, bool F16T>
 void launch_thin(SkinnyArgs a, const ThinPlan &p)
 {
-    if (p.splits == 1) a.ws = nullptr;
+    if (p.splits == 1 && a.halves == 1) a.ws = nullptr;
+    a.ksplits = p.splits;
     if (p.kw) {
         bool wide = false;                      // 16 thin rows: classifier heads only, which stream 16-bit activations
         if constexpr (SFMT == F16 || SFMT == BF16) {
@@ -1015,7 +1039,7 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
     } else {
         if (p.ct == 2) launch_thin_inst<SFMT, F16T, 1, 2>(a, p); else launch_thin_inst<SFMT, F16T, 1, 1>(a, p);
     }
-    if (p.splits > 1 && !tl_route.dry) {
+    if (a.ws && !tl_route.dry) {
         const uint64_t total = (uint64_t)a.NC * a.R;
         // four rows per thread where they are neighbours in the workspace and in C, and both are 16-byte aligned
         const bool vec = !a.mode_b && a.R % 4u == 0 && (reinterpret_cast<uintptr_t>(a.ws) & 15u) == 0 &&
@@ -1029,12 +1053,15 @@ template <int FMT, bool F16T>
 void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
 {
     const ThinPlan tp = plan_thin(FMT, M, L.N, L.K);
-    if (tp.use && (!tp.mode_b || ctx.w16) && (tp.splits == 1 || (uint64_t)tp.splits * tp.NC * tp.R <= ctx.ws_floats)) {
+    const uint32_t halves = tl_route.halves;
+    if (tp.use && (!tp.mode_b || ctx.w16) &&
+        ((tp.splits == 1 && halves == 1) || (uint64_t)tp.splits * halves * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
+        a.halves = halves; a.half_elems = (uint64_t)M * L.K;
         a.L = L; a.C = C; a.ws = ctx.ws; a.R = tp.R; a.NC = tp.NC; a.row_blocks = tp.row_blocks; a.cblocks = tp.cblocks; a.kper = tp.kper; a.out_f32 = out_f32; a.mode_b = tp.mode_b ? 1 : 0;
         tl_route.name = tp.kw ? "sp_skinny16_kw" : "sp_skinny16";
         if (tp.mode_b) {
-            if (ctx.soft_out && tp.kw && tp.splits == 1) {
+            if (ctx.soft_out && tp.kw && tp.splits == 1 && halves == 1) {
                 a.soft_out = ctx.soft_out;
                 a.soft_kind = ctx.soft_kind;
                 *ctx.soft_done = true;
@@ -1049,18 +1076,20 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         }
         return;
     }
-    GemmArgs g{L, A, C, M, out_f32, nullptr, 0};
+    GemmArgs g{L, A, C, M, out_f32, nullptr, 0, 1, halves};
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 8u == 0);
     const bool fits32 = (uint64_t)M * L.K * 2u < (1ull << 32) && (uint64_t)L.N * L.K * 2u < (1ull << 32);   // 32-bit DMA offsets
     // the 256 x 256 tiles need about a tile per compute unit; smaller problems fill the chip better with 128 x 128
     const uint32_t bm = gemm16_tile_rows(FMT, M, L.N);
     const uint32_t big_tiles = ((M + bm - 1) / bm) * ((L.N + 255u) / 256u);
     const uint32_t splits = gemm16_splits(FMT, M, L.N, L.K, &g.kper);
-    const bool split_ok = splits > 1 && (uint64_t)splits * M * L.N <= ctx.ws_floats;
-    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok)) {
+    const bool split_ok = splits > 1 && (uint64_t)splits * halves * M * L.N <= ctx.ws_floats;
+    const bool halves_ok = halves == 1 || (uint64_t)halves * M * L.N <= ctx.ws_floats;     // (checked by the caller's reserve)
+    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok) && halves_ok) {
         if (big_tiles >= 192u || !split_ok) g.kper = 0;
-        else g.ws = ctx.ws;
-        const dim3 grid(big_tiles, g.ws ? splits : 1u);
+        else g.ksplits = splits;
+        if (g.kper || halves == 2) g.ws = ctx.ws;
+        const dim3 grid(big_tiles, g.ksplits * halves);
         tl_route.name = "sp_gemm16_big";
         if (tl_route.dry) return;
         if (bm == 128u) {
@@ -1080,12 +1109,14 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         if (g.ws) {
             const uint64_t total = (uint64_t)M * L.N;
             const bool vec = L.N % 4u == 0 && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
-            if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, splits);
-            else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, splits);
+            if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, g.ksplits);
+            else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, g.ksplits);
         }
         return;
     }
     g.kper = 0;
+    g.ksplits = 1;
+    if (halves == 2) g.ws = ctx.ws;                  // one partial sum per activation matrix, added by the reduction
     tl_route.name = "sp_gemm16";
     if (tl_route.dry) return;
     // This kernel has one LDS stage, so it lives on the number of resident workgroups: the largest of 128 x 128,
@@ -1098,7 +1129,7 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const int shape = !(aligned || words) ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
     auto go = [&](auto tm_c, auto tn_c) {
         constexpr int TM = decltype(tm_c)::value, TN = decltype(tn_c)::value;
-        const uint32_t grid = tiles(64 * TM, 64 * TN);
+        const dim3 grid(tiles(64 * TM, 64 * TN), halves);
         if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
             if (words) {
                 sp_gemm16<FMT, F16T, TM, TN, true, true><<<grid, 256, 0, g_stream>>>(g);
@@ -1113,6 +1144,12 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     if (shape == 22) go(I2c{}, I2c{});
     else if (shape == 12) go(I1{}, I2c{});
     else go(I1{}, I1{});
+    if (g.ws) {
+        const uint64_t total = (uint64_t)M * L.N;
+        const bool vec = L.N % 4u == 0 && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+        if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, 1u);
+        else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, 1u);
+    }
 }
 
 void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
@@ -1179,7 +1216,9 @@ bool layer_wants_codes16(const sphip_net *net, uint32_t l /*1-based*/, uint32_t 
     return tp.use && tp.mode_b;
 }
 
-WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n)
+// halves = 2: a split-activation forward, in which every matrix-core layer writes one set of partial sums per
+// activation matrix
+WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t halves = 1)
 {
     WorkspaceNeed w{};
     w.act_floats = (uint64_t)n * net->max_width;
@@ -1201,10 +1240,10 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n)
         } else {
             const ThinPlan tp = plan_thin(net->prec, n, N, K);
             if (tp.use) {
-                if (tp.splits > 1) ws = (uint64_t)tp.splits * tp.NC * tp.R;
+                if (tp.splits > 1 || halves > 1) ws = (uint64_t)tp.splits * halves * tp.NC * tp.R;
             } else {
                 const uint32_t sp = gemm16_splits(net->prec, n, N, K, &kper);
-                if (sp > 1) ws = (uint64_t)sp * n * N;
+                if (sp > 1 || halves > 1) ws = (uint64_t)sp * halves * n * N;
             }
         }
         if (ws > w.split_floats) w.split_floats = ws;
@@ -1221,9 +1260,9 @@ void launch_codes16(int prec, const uint8_t *codes, uint16_t *out, uint64_t coun
 }
 
 // grows the net's own workspace to what n samples need
-int reserve(sphip_net *net, uint32_t n, bool keep_layers)
+int reserve(sphip_net *net, uint32_t n, bool keep_layers, uint32_t halves = 1)
 {
-    const WorkspaceNeed need = workspace_need(net, n);
+    const WorkspaceNeed need = workspace_need(net, n, halves);
     if (need.act_floats > net->cap_elems) {
         for (int i = 0; i < 2; ++i) {
             if (net->buf[i]) { HCHECK(hipFree(net->buf[i])); net->buf[i] = nullptr; }
@@ -1292,13 +1331,20 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
                     uint32_t only_layer, bool keep = false)
 {
     const Regime reg = pick_regime(net, n, flags);
+    // split activations: two FP16 matrices between the layers, whatever else the flags say
+    const bool split = (flags & SPHIP_SPLIT_ACTIVATIONS) && reg == R_GEMM16;
+    tl_route.halves = split ? 2u : 1u;
     // BF16 weights: FP16 activations against the FP16 copy of the weights unless BF16 activations are asked for
-    const bool wide = !(flags & SPHIP_BF16_ACTIVATIONS) && net->prec == BF16 && reg == R_GEMM16;
+    const bool wide = (split || !(flags & SPHIP_BF16_ACTIVATIONS)) && net->prec == BF16 && reg == R_GEMM16;
     const bool f16t = net->prec != BF16 || wide;  // 16-bit activation type of the matrix-core path
     const uint32_t last = net->layers - 1;
 
     const void *in = d_x;
-    if (reg == R_GEMM16 && !only_layer) {
+    if (split && !only_layer) {
+        const uint64_t cnt = (uint64_t)n * net->topo[0];
+        sp_cvt16_split<<<(uint32_t)((cnt + 255) / 256), 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
+        in = wk.buf[1];
+    } else if (reg == R_GEMM16 && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         const uint32_t grid = (uint32_t)((cnt / 4 + 255) / 256 + 1);
         if (f16t) sp_cvt16<true><<<grid, 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
@@ -1338,18 +1384,19 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
                 ctx.ws_floats = wk.split_cap;
                 if (softmax && !only_layer) {
                     ctx.soft_out = dst;
-                    ctx.soft_kind = !is_last ? (f16t ? 2 : 1) : 0;
+                    ctx.soft_kind = !is_last ? (split ? 3 : f16t ? 2 : 1) : 0;
                     ctx.soft_done = &soft_done;
                 }
                 launch_gemm16(wide ? (int)F16 : net->prec, L, (const uint16_t *)in, main_out, n, out_f32, ctx);
             }
         }
         if (softmax && !only_layer && !soft_done) {
-            const int kind = (reg == R_GEMM16 && !is_last) ? (f16t ? 2 : 1) : 0;
+            const int kind = (reg == R_GEMM16 && !is_last) ? (split ? 3 : f16t ? 2 : 1) : 0;
             sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(wk.soft_tmp, dst, kind, n, net->topo[l]);
         }
         in = dst;
     }
+    tl_route.halves = 1;
     HCHECK(hipGetLastError());
     return 0;
 }
@@ -1380,8 +1427,9 @@ uint32_t batch_block_rows(const sphip_net *net, uint32_t n, uint32_t flags)
 int reserve_batch(sphip_net *net, uint32_t n, uint32_t flags)
 {
     const uint32_t rows = batch_block_rows(net, n, flags);
-    if (reserve(net, rows, false)) return 1;
-    if (rows < n && n % rows != 0 && reserve(net, n % rows, false)) return 1;
+    const uint32_t halves = (flags & SPHIP_SPLIT_ACTIVATIONS) ? 2u : 1u;
+    if (reserve(net, rows, false, halves)) return 1;
+    if (rows < n && n % rows != 0 && reserve(net, n % rows, false, halves)) return 1;
     return 0;
 }
 
@@ -1618,7 +1666,7 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
 {
     if (!net || !x || !y || n == 0) return fail_msg("sphip_forward: invalid argument");
     if (check_uploaded(net)) return 1;
-    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH);
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH | SPHIP_SPLIT_ACTIVATIONS);
     if (reserve_batch(net, n, fwd_flags)) return 1;
     const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * net->topo[net->layers - 1];
     const float *d_x = x;
@@ -1667,7 +1715,7 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
         if (scratch_lookup(&base)) return 1;
     }
     // lay the workspace out inside the scratch array, every piece at a multiple of 256 bytes
-    const WorkspaceNeed need = workspace_need(net, n);
+    const WorkspaceNeed need = workspace_need(net, n, (flags & SPHIP_SPLIT_ACTIVATIONS) ? 2u : 1u);
     size_t used = 0;
     auto take = [&](uint64_t bytes) -> unsigned char * {
         unsigned char *p = base + used;
@@ -1689,7 +1737,7 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
     // an integer layer with few outputs reads an FP16 copy of its codes: the net's own if an earlier call made one,
     // else one made here, in the scratch array, on every call
     // (only the matrix-core regime reads them: a forced vector forward or one of up to four samples never does)
-    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS);
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_SPLIT_ACTIVATIONS);
     const bool reads_codes = pick_regime(net, n, fwd_flags) == R_GEMM16;
     bool fresh[kMaxLayers] = {};
     for (uint32_t l = 1; l < net->layers; ++l) {
@@ -1754,7 +1802,7 @@ int sphip_evaluate(sphip_net *net, const float *x, const float *targets, uint32_
     if (!net || !x || !targets || n == 0 || (loss_func != 0 && loss_func != 1))
         return fail_msg("sphip_evaluate: invalid argument");
     if (check_uploaded(net)) return 1;
-    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH);
+    const uint32_t fwd_flags = flags & (SPHIP_FORCE_GEMM | SPHIP_FORCE_GEMV | SPHIP_BF16_ACTIVATIONS | SPHIP_WHOLE_BATCH | SPHIP_SPLIT_ACTIVATIONS);
     if (reserve_batch(net, n, fwd_flags)) return 1;
     const uint32_t width = net->topo[net->layers - 1];
     const uint64_t in_cnt = (uint64_t)n * net->topo[0], out_cnt = (uint64_t)n * width;
@@ -1939,11 +1987,13 @@ const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, 
         ThinCtx ctx{};
         ctx.w16 = reinterpret_cast<const uint16_t *>(aligned_ptr);
         ctx.ws_floats = ~0ull;
+        tl_route.halves = (flags & SPHIP_SPLIT_ACTIVATIONS) ? 2u : 1u;
         launch_gemm16(net->prec, L, reinterpret_cast<const uint16_t *>(aligned_ptr), nullptr, n, 1, ctx);
         break;
     }
     }
     tl_route.dry = false;
+    tl_route.halves = 1;
     return tl_route.name;
 }
 

@@ -15,9 +15,26 @@ struct GemmArgs {
     void *C;               // [M][N] 16-bit, or FP32 when out_f32
     uint32_t M;
     int out_f32;
-    float *ws;             // [splits][M][N] partial sums when the grid splits K (sp_gemm16_big only), else nullptr
-    uint32_t kper;         // k range of one split, a multiple of 64 (0: all of K)
+    float *ws;             // [grid y][M][N] partial sums when grid y splits the product, else nullptr
+    uint32_t kper;         // k range of one K split, a multiple of 64 (0: all of K)
+    // Split activations: the layer input is two 16-bit matrices, hi and (a - hi) 2^11, the second M K elements
+    // behind the first; grid y = halves x ksplits, y / ksplits picks the matrix, y % ksplits the K range.
+    uint32_t ksplits;      // K splits (>= 1)
+    uint32_t halves;       // 1, or 2 with split activations
 };
+
+// 2^-11: what the partial sums of the second activation matrix are scaled by
+constexpr float kLoScale = 1.0f / 2048.0f;
+
+// hi and lo of a split activation: hi = v rounded to FP16, lo = (v - hi) 2^11 rounded to FP16 (v - hi is exact in FP32)
+__device__ __forceinline__ void split_f16(float v, uint16_t &hi, uint16_t &lo)
+{
+    hi = f32_to_f16_sat(v);
+    _Float16 hh;
+    __builtin_memcpy(&hh, &hi, 2);
+    const float rest = (v - (float)hh) * 2048.0f;
+    lo = (rest == rest && fabsf(rest) != __builtin_inff()) ? f32_to_f16_sat(rest) : (uint16_t)0;   // inf / NaN live in hi
+}
 
 // (float)q as a 16-bit float; exact for |q| <= 128 in either type
 template <bool F16T>
@@ -123,6 +140,7 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     const uint32_t M = g.M, N = g.L.N, K = g.L.K;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    const uint16_t *const A = g.A + (size_t)blockIdx.y * M * K;      // grid y > 1: the matrices of a split activation
 
     // tile index: consecutive workgroups go to different XCDs, so give each XCD a
     // contiguous band of tiles (shared A rows / W rows stay in one L2)
@@ -155,7 +173,7 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
                 const int c = t + 256 * i, row = c >> 3, kc = c & 7;
                 const uint32_t m = m0 + row < M ? m0 + row : M - 1;
                 const uint32_t k = k0 + kc * 8;
-                ra[i] = k < K ? *reinterpret_cast<const uint4 *>(g.A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
+                ra[i] = k < K ? *reinterpret_cast<const uint4 *>(A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
             }
             if constexpr (W4) {
 #pragma unroll
@@ -236,7 +254,7 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
             for (int e = t; e < BM * BK; e += 256) {
                 const int row = e / BK, kk = e % BK;
                 const uint32_t m = m0 + row, k = k0 + kk;
-                As[row * LDK + kk] = (m < M && k < K) ? g.A[(size_t)m * K + k] : (uint16_t)0;
+                As[row * LDK + kk] = (m < M && k < K) ? A[(size_t)m * K + k] : (uint16_t)0;
             }
             for (int e = t; e < BN * BK; e += 256) {
                 const int row = e / BK, kk = e % BK;
@@ -290,6 +308,21 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
         }
     }
 
+    if (g.ws) {                                        // partial sums of one activation matrix: a second launch adds them
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+            if (col >= N) continue;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (row < M) g.ws[((size_t)blockIdx.y * M + row) * N + col] = acc[i][j][r];
+                }
+        }
+        return;
+    }
     // epilogue: scale, bias, activation, store.  Sigmoid and tanh have a copy of the loops to themselves: a switch
     // over all activations behind every one of a lane's outputs is mostly their code, fetched for nothing.
     const float wscale = g.L.wscale;
@@ -446,7 +479,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     // the rows of two of its loads are a multiple of 16 apart
     static_assert(NWAVES % 2 == 0 && HALF % 2 == 0, "the swizzle of a lane's loads must not depend on the load");
     const uint32_t kchunk = (uint32_t)((lane & 7) ^ ((((wave & (HALF - 1)) * 8 + (lane >> 3)) >> 1) & 7)) << 3;
-    const char *a_base = reinterpret_cast<const char *>(g.A);
+    const char *a_base = reinterpret_cast<const char *>(g.A + (size_t)(blockIdx.y / g.ksplits) * g.M * g.L.K);
     const char *w_base = reinterpret_cast<const char *>(g.L.w);
     const size_t w_row_bytes = (size_t)K * bits / 8u;
     uint4 rw[W_LOADS];
@@ -621,7 +654,7 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     };
 
     // grid y splits K for problems with too few tiles to fill the chip
-    const uint32_t kbeg = g.kper ? blockIdx.y * g.kper : 0u;
+    const uint32_t kbeg = g.kper ? (blockIdx.y % g.ksplits) * g.kper : 0u;
     const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
     const uint32_t ktiles = (kend - kbeg + BK - 1) / BK;
     const uint32_t tail = (kend - kbeg) % BK;              // only the last K split can have one
@@ -761,23 +794,27 @@ __global__ __launch_bounds__(64 * WM * WN) void sp_gemm16_big(const GemmArgs g)
     }
 }
 
-// adds the K splits of sp_gemm16_big (in split order) and applies scale, bias and activation
-// adds the K splits of sp_gemm16_big and applies scale, bias and activation; a thread takes four neighbouring
-// columns (VEC: N a multiple of four, workspace and C 16-byte aligned) or one
+// adds the partial sums of a split launch (K splits in split order; with split activations the sums of the second
+// matrix, scaled by 2^-11, after those of the first) and applies scale, bias and activation; a thread takes four
+// neighbouring columns (VEC: N a multiple of four, workspace and C 16-byte aligned) or one.  16-bit outputs of a
+// split-activation forward are written as the two matrices of the next layer's input (g.halves == 2).
 template <bool F16T, bool VEC>
 __global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32_t splits)
 {
     const uint64_t total = (uint64_t)g.M * g.L.N;
+    const uint32_t parts = splits * g.halves;
     if constexpr (VEC) {
         const uint64_t idx = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
         if (idx >= total) return;
-        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        for (uint32_t sp = 0; sp < splits; ++sp) {
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f), low = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (uint32_t sp = 0; sp < parts; ++sp) {
             const float4 v = *reinterpret_cast<const float4 *>(g.ws + (uint64_t)sp * total + idx);
-            sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            if (sp < splits) { sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w; }
+            else { low.x += v.x; low.y += v.y; low.z += v.z; low.w += v.w; }
         }
         const uint32_t col = (uint32_t)(idx % g.L.N);
-        const float in[4] = {sum.x, sum.y, sum.z, sum.w};
+        const float in[4] = {fmaf(low.x, kLoScale, sum.x), fmaf(low.y, kLoScale, sum.y), fmaf(low.z, kLoScale, sum.z),
+                             fmaf(low.w, kLoScale, sum.w)};
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -786,6 +823,13 @@ __global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32
         }
         if (g.out_f32) {
             *reinterpret_cast<float4 *>(reinterpret_cast<float *>(g.C) + idx) = make_float4(v[0], v[1], v[2], v[3]);
+        } else if (g.halves == 2) {
+            uint16_t hi[4], lo[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) split_f16(v[i], hi[i], lo[i]);
+            uint16_t *c = reinterpret_cast<uint16_t *>(g.C);
+            *reinterpret_cast<uint2 *>(c + idx) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16));
+            *reinterpret_cast<uint2 *>(c + total + idx) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
         } else {
             const uint32_t lo = (uint32_t)f32_to_t16<F16T>(v[0]) | ((uint32_t)f32_to_t16<F16T>(v[1]) << 16);
             const uint32_t hi = (uint32_t)f32_to_t16<F16T>(v[2]) | ((uint32_t)f32_to_t16<F16T>(v[3]) << 16);
@@ -794,12 +838,20 @@ __global__ __launch_bounds__(256) void sp_gemm16_reduce(const GemmArgs g, uint32
     } else {
         const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
         if (idx >= total) return;
-        float sum = 0.0f;
-        for (uint32_t sp = 0; sp < splits; ++sp) sum += g.ws[(uint64_t)sp * total + idx];
+        float sum = 0.0f, low = 0.0f;
+        for (uint32_t sp = 0; sp < parts; ++sp) {
+            const float v = g.ws[(uint64_t)sp * total + idx];
+            if (sp < splits) sum += v; else low += v;
+        }
         const uint32_t col = (uint32_t)(idx % g.L.N);
         const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
-        const float v = apply_act(fmaf(sum, g.L.wscale, bias), g.L.act);
+        const float v = apply_act(fmaf(fmaf(low, kLoScale, sum), g.L.wscale, bias), g.L.act);
         if (g.out_f32) reinterpret_cast<float *>(g.C)[idx] = v;
-        else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
+        else if (g.halves == 2) {
+            uint16_t hi, lo;
+            split_f16(v, hi, lo);
+            reinterpret_cast<uint16_t *>(g.C)[idx] = hi;
+            reinterpret_cast<uint16_t *>(g.C)[total + idx] = lo;
+        } else reinterpret_cast<uint16_t *>(g.C)[idx] = f32_to_t16<F16T>(v);
     }
 }

@@ -29,6 +29,11 @@ struct SkinnyArgs {
     int mode_b;              // 0: streamed rows are outputs, thin rows samples; 1: the reverse
     void *soft_out;          // sp_skinny16_kw, mode_b, no K split: softmax over a sample's outputs goes here instead of C
     int soft_kind;           // its element type: 0 FP32, 1 BF16, 2 FP16
+    // Split activations (GemmArgs has the layout): grid y = halves x ksplits, y / ksplits picks the activation matrix
+    // (the thin operand, or the streamed one in mode b), y % ksplits the K range.
+    uint32_t ksplits;        // K splits (>= 1)
+    uint32_t halves;         // 1, or 2 with split activations
+    uint64_t half_elems;     // elements between the two activation matrices (samples x K)
 };
 
 template <int FMT>
@@ -175,7 +180,10 @@ __global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
     }
     const uint32_t row0 = (rblk * (uint32_t)NWV + (uint32_t)wave) * (32u * RT);
     const uint32_t cbase = cblk * (32u * CT);
-    const uint32_t kbeg = blockIdx.y * a.kper;
+    const uint32_t half = blockIdx.y / a.ksplits;
+    const uint8_t *const stream = a.mode_b ? a.stream + (size_t)half * a.half_elems * 2u : a.stream;
+    const uint16_t *const thin = a.mode_b ? a.thin : a.thin + (size_t)half * a.half_elems;
+    const uint32_t kbeg = (blockIdx.y % a.ksplits) * a.kper;
     const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
     const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
     const size_t row_bytes = (size_t)K * F::bits / 8u;
@@ -215,7 +223,7 @@ __global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
     const uint32_t last_chunk = nchunks - 1;
     auto issue_stream = [&](uint32_t ch, u32x4 (&dst)[RT][LPC]) {
         if (ch < last_chunk) {
-            const uint8_t *sb = a.stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
+            const uint8_t *sb = stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
 #pragma unroll
             for (int i = 0; i < LPC; ++i)
 #pragma unroll
@@ -232,14 +240,14 @@ __global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
                 const uint32_t k = kc0 + 2u * i * EPL;                 // first code of the h = 0 lane load
                 const uint32_t add = k + h * EPL < K ? k * F::bits / 8u : 0u - h * 16u;
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) load16_async<0>(dst[rt][i], svoff[rt] + add, a.stream);
+                for (int rt = 0; rt < RT; ++rt) load16_async<0>(dst[rt][i], svoff[rt] + add, stream);
             }
         }
     };
     u32x4 thin_regs[UPT][2];
     auto issue_thin = [&](uint32_t ch) {
         if (ch < last_chunk) {
-            const uint16_t *tb = a.thin + (kbeg + ch * BKC);
+            const uint16_t *tb = thin + (kbeg + ch * BKC);
 #pragma unroll
             for (int q = 0; q < UPT; ++q)
 #pragma unroll
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(64 * NWV) void sp_skinny16(const SkinnyArgs a)
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     const bool valid = trow_ok[q] && kc0 + uc * 16u + 8u * e + 8u <= kend;
-                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, a.thin);
+                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, thin);
                 }
             }
         }
@@ -419,7 +427,10 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     const uint32_t n31 = lane & 31, h = lane >> 5;
     const uint32_t K = a.L.K;
     const uint32_t r_out = blockIdx.x * 32u + n31;
-    const uint32_t kbeg = blockIdx.y * a.kper;
+    const uint32_t half = blockIdx.y / a.ksplits;
+    const uint8_t *const stream = a.mode_b ? a.stream + (size_t)half * a.half_elems * 2u : a.stream;
+    const uint16_t *const thin = a.mode_b ? a.thin : a.thin + (size_t)half * a.half_elems;
+    const uint32_t kbeg = (blockIdx.y % a.ksplits) * a.kper;
     const uint32_t kend = kbeg + a.kper < K ? kbeg + a.kper : K;
     const uint32_t nchunks = (kend - kbeg + BKC - 1) / BKC;
     const size_t row_bytes = (size_t)K * F::bits / 8u;
@@ -449,7 +460,7 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     auto issue_stream = [&](uint32_t i, u32x4 (&dst)[LPC]) {
         const uint32_t ch = chunk_of(i);
         if (ch < last_chunk) {
-            const uint8_t *sb = a.stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
+            const uint8_t *sb = stream + (size_t)(kbeg + ch * BKC) * F::bits / 8u;
 #pragma unroll
             for (int j = 0; j < LPC; ++j) {
                 if (j == 0) load16_async<0>(dst[j], svoff, sb);
@@ -463,7 +474,7 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
             for (int j = 0; j < LPC; ++j) {
                 const uint32_t k = kc0 + 2u * j * EPL;                 // first code of the h = 0 lane load
                 const uint32_t add = k + h * EPL < K ? k * F::bits / 8u : 0u - h * 16u;
-                load16_async<0>(dst[j], svoff + add, a.stream);
+                load16_async<0>(dst[j], svoff + add, stream);
             }
         }
     };
@@ -471,7 +482,7 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     auto issue_thin = [&](uint32_t i) {
         const uint32_t ch = chunk_of(i);
         if (ch < last_chunk) {
-            const uint16_t *tb = a.thin + (kbeg + ch * BKC);
+            const uint16_t *tb = thin + (kbeg + ch * BKC);
 #pragma unroll
             for (int q = 0; q < UPL; ++q)
 #pragma unroll
@@ -484,7 +495,7 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     const bool valid = trow_ok[q] && kc0 + uc * 16u + 8u * e + 8u <= kend;
-                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, a.thin);
+                    load16_async<0>(thin_regs[q][e], valid ? tvoff[q][e] + kc0 * 2u : 0u, thin);
                 }
             }
         }
@@ -630,22 +641,39 @@ __global__ __launch_bounds__(64 * NW) void sp_skinny16_kw(const SkinnyArgs a)
     }
 }
 
-// adds the K splits of sp_skinny16 and applies bias and activation; a thread takes four neighbouring streamed rows
-// (VEC: R is a multiple of four and the rows are outputs, so they are neighbours in C as well) or one
+// adds the partial sums of sp_skinny16 (K splits in split order; with split activations the sums of the second matrix,
+// scaled by 2^-11, after those of the first) and applies bias and activation; a thread takes four neighbouring
+// streamed rows (VEC: R is a multiple of four and the rows are outputs, so they are neighbours in C as well) or one
+template <bool F16T>
+__device__ __forceinline__ void skinny_store(const SkinnyArgs &a, size_t o, float v)
+{
+    if (a.out_f32) reinterpret_cast<float *>(a.C)[o] = v;
+    else if (a.halves == 2) {
+        uint16_t hi, lo;
+        split_f16(v, hi, lo);
+        uint16_t *c = reinterpret_cast<uint16_t *>(a.C);
+        c[o] = hi;
+        c[(size_t)a.NC * a.R + o] = lo;               // samples x outputs elements further on
+    } else reinterpret_cast<uint16_t *>(a.C)[o] = f32_to_t16<F16T>(v);
+}
+
 template <bool F16T, bool VEC>
 __global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint32_t splits)
 {
     const uint64_t total = (uint64_t)a.NC * a.R;
+    const uint32_t parts = splits * a.halves;
     if constexpr (VEC) {
         const uint64_t idx = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
         if (idx >= total) return;
-        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        for (uint32_t sp = 0; sp < splits; ++sp) {
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f), low = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (uint32_t sp = 0; sp < parts; ++sp) {
             const float4 v = *reinterpret_cast<const float4 *>(a.ws + (uint64_t)sp * total + idx);
-            sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            if (sp < splits) { sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w; }
+            else { low.x += v.x; low.y += v.y; low.z += v.z; low.w += v.w; }
         }
         const uint32_t c = (uint32_t)(idx / a.R), r = (uint32_t)(idx % a.R);
-        const float in[4] = {sum.x, sum.y, sum.z, sum.w};
+        const float in[4] = {fmaf(low.x, kLoScale, sum.x), fmaf(low.y, kLoScale, sum.y), fmaf(low.z, kLoScale, sum.z),
+                             fmaf(low.w, kLoScale, sum.w)};
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -655,6 +683,13 @@ __global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint
         const size_t o = (size_t)c * a.L.N + r;
         if (a.out_f32) {
             *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.C) + o) = make_float4(v[0], v[1], v[2], v[3]);
+        } else if (a.halves == 2) {
+            uint16_t hi[4], lo[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) split_f16(v[i], hi[i], lo[i]);
+            uint16_t *cc = reinterpret_cast<uint16_t *>(a.C);
+            *reinterpret_cast<uint2 *>(cc + o) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16));
+            *reinterpret_cast<uint2 *>(cc + total + o) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
         } else {
             const uint32_t lo = (uint32_t)f32_to_t16<F16T>(v[0]) | ((uint32_t)f32_to_t16<F16T>(v[1]) << 16);
             const uint32_t hi = (uint32_t)f32_to_t16<F16T>(v[2]) | ((uint32_t)f32_to_t16<F16T>(v[3]) << 16);
@@ -663,9 +698,15 @@ __global__ __launch_bounds__(256) void sp_skinny_reduce(const SkinnyArgs a, uint
     } else {
         const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
         if (idx >= total) return;
-        float sum = 0.0f;
-        for (uint32_t sp = 0; sp < splits; ++sp) sum += a.ws[(uint64_t)sp * total + idx];
-        skinny_emit<F16T>(a, (uint32_t)(idx / a.R), (uint32_t)(idx % a.R), sum);
+        float sum = 0.0f, low = 0.0f;
+        for (uint32_t sp = 0; sp < parts; ++sp) {
+            const float v = a.ws[(uint64_t)sp * total + idx];
+            if (sp < splits) sum += v; else low += v;
+        }
+        const uint32_t c = (uint32_t)(idx / a.R), r = (uint32_t)(idx % a.R);
+        const uint32_t m = a.mode_b ? r : c, n = a.mode_b ? c : r;
+        const float bias = elem_value_rt(a.L.bias_fmt, a.L.bias, n) * a.L.bscale;
+        skinny_store<F16T>(a, (size_t)m * a.L.N + n, apply_act(fmaf(fmaf(low, kLoScale, sum), a.L.wscale, bias), a.L.act));
     }
 }
 

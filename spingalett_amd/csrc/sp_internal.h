@@ -32,6 +32,7 @@ typedef struct {
     sp_packed_array *packed_b;      /* [layers-1] */
     bool             opt_loaded;    /* opt_m / opt_v / grad_* may hold content: a file's optimizer block was read
                                        into them, or train() copied the device's gradients and moments back */
+    int              act_mode;      /* SpingalettNetActivations: this net's own choice of activation type */
     /* device side */
     sphip_net       *dev;
     PrecisionMode    dev_precision;
