@@ -198,11 +198,19 @@ def timed_layer(copies, l, n, iters, flags=0):
 
 
 def roofline_for(copies, topo, prec, n, iters):
-    """Times the main kernel of the largest layer alone (HIP events on its stream)."""
+    """Times the main kernel of the largest layer alone (HIP events on its stream).  A net with several layers of that
+    shape (the same kernel, the same launch) reports their average, as a profiler's per-kernel average does: the
+    duration depends on the operand values (the part's clock under this load follows how many bits toggle), and the
+    first such layer sees the raw inputs, the others activations."""
     l = dominant_layer(topo)
-    ms = timed_layer(copies, l, n, iters)
     K, N = topo[l - 1], topo[l]
+    same = [i for i in range(1, len(topo)) if (topo[i - 1], topo[i]) == (K, N)]
+    ms = float(np.mean([timed_layer(copies, i, n, iters) for i in same]))
     kernel = S.lib().sphip_layer_kernel_name(copies[0].h, l, n, 0).decode()
+    # a batch that runs in blocks of rows launches the layer's kernel once per block: ms (and traffic) are those of
+    # all of them together, the layer's share of one forward
+    rows = S.lib().sphip_batch_block_rows(copies[0].h, n, 0)
+    launches = -(-n // rows) if rows else 1
     traffic = PROFILED_TRAFFIC.get((kernel, (n, N, K)))
     if traffic is None:
         print(f"bench.py: no profiled traffic for {kernel} at [n, N, K] = {[n, N, K]} in profiles/traffic.json "
@@ -212,12 +220,12 @@ def roofline_for(copies, topo, prec, n, iters):
         nbytes = array_payload(K * N, prec) + array_payload(N, prec) + 4 * n * (K + N)
         ach = nbytes / (ms * 1e-3)
         return dict(bound="hbm", achieved=ach / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s", frac=ach / HBM_PEAK,
-                    traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+                    traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms, launches=launches)
     fl = 2.0 * n * K * N
     ach = fl / (ms * 1e-3)
     peak = FP32_PEAK if prec == S.PRECISION_FLOAT32 else MFMA16_PEAK
     return dict(bound="mfma", achieved=ach / 1e12, peak=peak / 1e12, unit="TFLOP/s", frac=ach / peak,
-                traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms)
+                traffic=traffic, kernel=kernel, layer=l, shape=[n, N, K], avg_ms=ms, launches=launches)
 
 
 def cpu_baseline(path, cfg, n_sample, budget_s=12.0):
@@ -277,7 +285,7 @@ def cpu_baseline_single(path, cfg, budget_s=2.0):
                 sample=f"one sample, the public forward's call sequence, {blas_short(desc)} sgemv and OpenMP dot rows")
 
 
-def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0.0):
+def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0.0, alternatives=True):
     cfg = WORKLOADS[name]
     topo, prec = cfg["topo"], cfg["prec"]
     t0 = time.perf_counter()
@@ -297,7 +305,7 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
                    copies=len(copies), finite=bool(np.isfinite(y).all()))
         if n in cfg.get("roofline_batches", batches):
             row["roofline"] = roofline_for(copies, topo, prec, n, 20 if n >= 1024 else 200)
-        if prec == S.PRECISION_BFLOAT16 and n >= 5:
+        if alternatives and prec == S.PRECISION_BFLOAT16 and n >= 5:
             # the same workload with BF16 activations on the BF16 matrix cores (SPHIP_BF16_ACTIVATIONS /
             # spingalett_set_bf16_activations): the faster, less accurate setting; the figures above are the default's
             # (FP16 activations against the FP16 copy of the BF16 weights)
@@ -308,7 +316,7 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
             row["bf16_activations"] = dict(ms_per_step=w_wall, samples_per_s=n / (w_wall * 1e-3),
                                            mfma_frac=fl / (w_ev * 1e-3) / MFMA16_PEAK, dominant_layer_ms=w_layer,
                                            dominant_layer_frac=2.0 * n * topo[l - 1] * topo[l] / (w_layer * 1e-3) / MFMA16_PEAK)
-        if want_output and prec != S.PRECISION_FLOAT32 and n >= 5:
+        if alternatives and want_output and prec != S.PRECISION_FLOAT32 and n >= 5:
             # the same workload with split activations (SPHIP_SPLIT_ACTIVATIONS / spingalett_set_net_activations): two
             # FP16 numbers per activation, twice the matrix-core work, FP32-grade outputs; the opt-in setting that
             # meets 99.9 % argmax agreement on 1000-class heads.  Fractions are of the algorithmic flops, not of the
@@ -375,6 +383,8 @@ def compact_row(row):
     if rl:
         out["dom"] = dict(k=rl["kernel"], l=rl["layer"], bound=rl["bound"], frac=rl["frac"], ms=rl["avg_ms"],
                           traffic=rl["traffic"])
+        if rl["launches"] > 1:
+            out["dom"]["launches"] = rl["launches"]
     if "public_forward_us" in row:
         out["fwd_us"] = row["public_forward_us"]
     if "cpu_baseline_b1" in row:
@@ -447,6 +457,30 @@ def run_training(steps, warmup, cpu=True):
     return out
 
 
+def vendor_gemm(m, steps, warmup):
+    """Speed-of-light comparison, not part of the product: the vendor library's 16-bit GEMM (torch.matmul ->
+    hipBLASLt) on an m x m x m product of BF16 operands with this benchmark's value distribution (N(0,1) activations,
+    N(0, 2/m) weights), timed with events after the same 50 ms of warm-up launches as the library's own layers."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(42)
+    a = torch.randn((m, m), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((m, m), generator=g, device="cuda", dtype=torch.float32) * (2.0 / m) ** 0.5).to(torch.bfloat16)
+    c = torch.empty((m, m), device="cuda", dtype=torch.bfloat16)
+    for _ in range(max(warmup, 60)):
+        torch.matmul(a, w.t(), out=c)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        torch.matmul(a, w.t(), out=c)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    fl = 2.0 * m * m * m
+    return dict(kernel="torch.matmul (hipBLASLt), BF16", shape=[m, m, m], avg_ms=ms, frac=fl / (ms * 1e-3) / MFMA16_PEAK,
+                achieved_tflops=fl / (ms * 1e-3) / 1e12)
+
+
 def release(w):
     for hc in w["clones"]:
         S.lib().sphip_destroy(hc)
@@ -468,10 +502,20 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="headline batch (default: the workload's largest)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations and the training benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-alt", action="store_true",
+                    help="skip the headline workload's alternative activation settings (BF16 activations, split "
+                         "activations), so that a profile holds the default setting's launches only")
+    ap.add_argument("--vendor-gemm", type=int, default=0, metavar="M",
+                    help="instead of a workload, time the vendor library's BF16 GEMM on an M x M x M product (needs torch; "
+                         "a comparison for the profiles, not part of the product)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also make one device-to-device copy of the net's arrays (a plain copy kernel of known "
                          "size, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
+    if args.vendor_gemm:
+        # before anything of this library touches the GPU: torch brings its own copy of the HIP runtime
+        print(json.dumps(sig(vendor_gemm(args.vendor_gemm, args.steps, args.warmup))))
+        return 0
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         return 2
@@ -494,7 +538,7 @@ def main():
         return 0
     cfg = WORKLOADS[args.workload]
     n = args.batch or max(cfg["batches"])
-    head = run_workload(args.workload, [n], args.steps, args.warmup, want_output=True)
+    head = run_workload(args.workload, [n], args.steps, args.warmup, want_output=True, alternatives=not args.no_alt)
     row = head["rows"][0]
     if args.calibrate_copy:
         hc = C.c_void_p()
@@ -543,7 +587,7 @@ def main():
         "config": {"workload": f"{args.workload}: {'->'.join(map(str, cfg['topo']))} {row['format']} weights, batch {n}",
                    "format": row["format"], "batch": n},
         "roofline": {k: rl[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
-        "roofline_kernel": {k: rl[k] for k in ("kernel", "layer", "shape", "avg_ms")},
+        "roofline_kernel": {k: rl[k] for k in ("kernel", "layer", "shape", "avg_ms", "launches")},
         "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
         "bf16_activations": row.get("bf16_activations"),
         "split_activations": row.get("split_activations"),

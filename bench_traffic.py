@@ -10,8 +10,8 @@
 FETCH_SIZE / WRITE_SIZE are read per dispatch.  The dispatches of the dominant layer are those of the named kernel
 whose reading is within 20 % of that kernel's largest (the other layers of the net are smaller).  Each counter is scaled
 by what it reads for the plain copy of the net's largest array that --calibrate-copy makes in the same run (a copy
-kernel reads and writes exactly that many bytes).  bytes = fetch + write of one launch, what bench.py reports as
-roofline.traffic.  No GPU is needed to run this script.
+kernel reads and writes exactly that many bytes).  bytes = fetch + write of one launch (times --launches for a batch that
+runs in blocks of rows), what bench.py reports as roofline.traffic.  No GPU is needed to run this script.
 """
 from __future__ import annotations
 
@@ -61,6 +61,9 @@ def main():
     ap.add_argument("--kernel", required=True, help="name as sphip_layer_kernel_name reports it")
     ap.add_argument("--fetch", required=True, help="directory of the FETCH_SIZE run")
     ap.add_argument("--write", required=True, help="directory of the WRITE_SIZE run")
+    ap.add_argument("--launches", type=int, default=1,
+                    help="launches of the kernel per forward of the layer (a batch that runs in blocks of rows: bench.py "
+                         "reports it as roofline_kernel.launches); the entry holds their sum")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles", "traffic.json"))
     args = ap.parse_args()
 
@@ -83,13 +86,14 @@ def main():
         "fetch_per_dispatch": round(fetch, 1), "write_per_dispatch": round(write, 1), "dispatches_averaged": nf,
         "fetch_factor_kib": round(f_factor, 4), "write_factor_kib": round(w_factor, 4),
         "calibration_copy_bytes": copy_bytes,
-        "bytes": int(round((fetch * f_factor + write * w_factor) * 1024)),
+        "launches_per_forward": args.launches,
+        "bytes": int(round((fetch * f_factor + write * w_factor) * 1024)) * args.launches,
         "commands": [
             f"rocprofv3 --pmc {c} -d out/{d} -o p --output-format csv -- python3 bench.py --workload {args.workload} "
             f"--batch {args.batch} --steps 40 --warmup 5 --no-extra --no-cpu --calibrate-copy"
             for c, d in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write"))
         ] + [f"python3 bench_traffic.py --workload {args.workload} --batch {args.batch} --kernel {args.kernel} "
-             "--fetch out/fetch --write out/write"],
+             "--fetch out/fetch --write out/write" + (f" --launches {args.launches}" if args.launches > 1 else "")],
     }
     try:
         with open(args.out) as f:

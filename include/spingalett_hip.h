@@ -183,6 +183,9 @@ SPHIP_API int  sphip_time_layer(sphip_net *const *nets, int count, uint32_t laye
 /* `iters` training steps on device-resident inputs and targets, timed like sphip_time_forward. */
 SPHIP_API int  sphip_time_train_step(sphip_net *net, const float *d_x, const float *d_targets, uint32_t n,
                                      const sphip_train_args *args, int iters, float *ms);
+/* Rows per pass of a forward of n samples with these flags: n, or the block size when the batch runs in blocks of rows
+ * (SPHIP_WHOLE_BATCH has the rule); every layer kernel is then launched once per block. */
+SPHIP_API uint32_t sphip_batch_block_rows(sphip_net *net, uint32_t n, uint32_t flags);
 /* Name of the main kernel that a forward of n samples with these flags runs for the given layer (1..layers-1):
  * the library's routing evaluated without launching anything. */
 SPHIP_API const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n,

@@ -142,7 +142,7 @@ SPHIP_SYMBOLS = [
     "sphip_forward", "sphip_forward_noalloc", "sphip_forward_layers", "sphip_decode", "sphip_synchronize", "sphip_malloc", "sphip_free",
     "sphip_device_memory",
     "sphip_memcpy_h2d", "sphip_memcpy_d2h", "sphip_clone", "sphip_time_forward", "sphip_time_layer",
-    "sphip_layer_kernel_name", "sphip_evaluate",
+    "sphip_layer_kernel_name", "sphip_batch_block_rows", "sphip_evaluate",
     "sphip_train_begin", "sphip_train_end", "sphip_train_set", "sphip_train_get", "sphip_train_step",
     "sphip_time_train_step",
 ]
@@ -238,6 +238,7 @@ def lib():
     L.sphip_time_layer.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int,
                                    C.POINTER(C.c_float)]
     L.sphip_time_layer.restype = C.c_int
+    L.sphip_batch_block_rows.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32]; L.sphip_batch_block_rows.restype = C.c_uint32
     L.sphip_layer_kernel_name.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32]
     L.sphip_layer_kernel_name.restype = C.c_char_p
     L.sphip_train_begin.argtypes = [C.c_void_p]; L.sphip_train_begin.restype = C.c_int

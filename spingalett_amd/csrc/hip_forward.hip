@@ -20,6 +20,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -502,6 +503,14 @@ __global__ __launch_bounds__(256) void sp_pack_layers(const PackArgs a)
         a.dst[a.dst_off[s] + i] = a.src[a.src_off[s] + i];
 }
 
+// The last launch of a single-sample forward: a sequence number into pinned host memory, system scope, behind the
+// kernel boundary that made the gathered activations visible.  The host polls the word instead of asking the runtime
+// to wait for the stream.
+__global__ __launch_bounds__(64) void sp_signal_host(uint32_t *flag, uint32_t seq)
+{
+    if (threadIdx.x == 0) __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // ---------------------------------------------------------------------------
 // evaluation of a batch of outputs (compute_sample_loss, SIMD.c:522-552;
 // batch_compute_loss, Training.c:421-435): one wave per sample
@@ -634,6 +643,8 @@ struct sphip_net {
     std::vector<uint32_t> slot_off;  // start of each layer's slot (floats)
     uint64_t slots_total = 0;
     float *pin_in = nullptr, *pin_out = nullptr;   // pinned host staging of small inputs / outputs
+    uint32_t *pin_flag = nullptr;  // pinned word the last launch of a single-sample forward writes its sequence number to
+    uint32_t flag_seq = 0;
     uint64_t pin_in_cap = 0, pin_out_cap = 0;
     float *stage_x = nullptr;      // device staging of host inputs / outputs
     float *stage_y = nullptr;
@@ -1515,6 +1526,7 @@ void sphip_destroy(sphip_net *net)
     if (net->layers_buf) (void)hipFree(net->layers_buf);
     if (net->pin_in) (void)hipHostFree(net->pin_in);
     if (net->pin_out) (void)hipHostFree(net->pin_out);
+    if (net->pin_flag) (void)hipHostFree(net->pin_flag);
     if (net->stage_x) (void)hipFree(net->stage_x);
     if (net->stage_y) (void)hipFree(net->stage_y);
     delete net;
@@ -1584,6 +1596,30 @@ int sphip_clone(const sphip_net *src, sphip_net **out)
     }
     HCHECK(hipStreamSynchronize(g_stream));
     *out = net;
+    return 0;
+}
+
+// Waits until everything enqueued so far has finished, for calls whose results are a few values in pinned host
+// memory: a last one-wave launch stores the call's sequence number into a pinned word and the host polls it (the
+// runtime's own wait costs several microseconds after the last kernel has ended).  Bounded: after about 50 ms
+// without the number the stream is waited for in the ordinary way, which also reports a failed kernel.
+static int wait_for_small_results(sphip_net *net)
+{
+    if (!net->pin_flag) {
+        HCHECK(hipHostMalloc((void **)&net->pin_flag, 64, hipHostMallocDefault));
+        *net->pin_flag = 0;
+    }
+    const uint32_t seq = ++net->flag_seq ? net->flag_seq : ++net->flag_seq;     // never 0
+    sp_signal_host<<<1, 64, 0, g_stream>>>(net->pin_flag, seq);
+    HCHECK(hipGetLastError());
+    const volatile uint32_t *flag = net->pin_flag;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spin = 1;; ++spin) {
+        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return 0;
+        __builtin_ia32_pause();
+        if ((spin & 0xFFFu) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(50)) break;
+    }
+    HCHECK(hipStreamSynchronize(g_stream));
     return 0;
 }
 
@@ -1695,9 +1731,13 @@ int sphip_forward(sphip_net *net, const float *x, uint32_t n, float *y, uint32_t
     }
     if (enqueue_forward_batch(net, d_x, n, d_y, fwd_flags, 0)) return 1;
     if (!(flags & SPHIP_Y_ON_DEVICE)) {
-        if (!y_pinned) HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
-        HCHECK(hipStreamSynchronize(g_stream));
-        if (y_pinned) memcpy(y, net->pin_out, out_cnt * sizeof(float));
+        if (y_pinned) {
+            if (wait_for_small_results(net)) return 1;
+            memcpy(y, net->pin_out, out_cnt * sizeof(float));
+        } else {
+            HCHECK(hipMemcpyAsync(y, d_y, out_cnt * sizeof(float), hipMemcpyDeviceToHost, g_stream));
+            HCHECK(hipStreamSynchronize(g_stream));
+        }
     }
     return 0;
 }
@@ -1790,8 +1830,7 @@ int sphip_forward_layers(sphip_net *net, const float *x, float *host_neurons)
         if (gx > 64) gx = 64;
         sp_pack_layers<<<dim3(gx, pa.count), 256, 0, g_stream>>>(pa);
     }
-    HCHECK(hipGetLastError());
-    HCHECK(hipStreamSynchronize(g_stream));
+    if (wait_for_small_results(net)) return 1;
     memcpy(host_neurons, net->pin_out, net->total_neurons * sizeof(float));
     return 0;
 }
@@ -1965,6 +2004,12 @@ int sphip_time_layer(sphip_net *const *nets, int count, uint32_t layer, uint32_t
         if (grow(&nets[i]->stage_x, &nets[i]->stage_x_cap, (uint64_t)n * nets[i]->topo[0])) return 1;
     }
     return time_common(nets, count, nets[0]->stage_x, n, nets[0]->stage_y, flags, iters, ms, layer);
+}
+
+uint32_t sphip_batch_block_rows(sphip_net *net, uint32_t n, uint32_t flags)
+{
+    if (!net || n == 0) return 0;
+    return batch_block_rows(net, n, flags);
 }
 
 const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, uint32_t flags)
