@@ -437,15 +437,23 @@ __global__ __launch_bounds__(256) void sp_cvt16(const float *__restrict__ in, ui
 // elements further on (the difference is exact in FP32; infinities and NaNs live in hi alone)
 __global__ __launch_bounds__(256) void sp_cvt16_split(const float *__restrict__ in, uint16_t *__restrict__ out, uint64_t n)
 {
-    const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-    if (i >= n) return;
-    const float v = in[i];
-    const uint16_t hi = f32_to_f16_sat(v);
-    _Float16 hh;
-    __builtin_memcpy(&hh, &hi, 2);
-    const float rest = (v - (float)hh) * 2048.0f;
-    out[i] = hi;
-    out[n + i] = (rest == rest && fabsf(rest) != __builtin_inff()) ? f32_to_f16_sat(rest) : (uint16_t)0;
+    auto one = [](float v, uint16_t &hi, uint16_t &lo) {
+        hi = f32_to_f16_sat(v);
+        _Float16 hh;
+        __builtin_memcpy(&hh, &hi, 2);
+        const float rest = (v - (float)hh) * 2048.0f;
+        lo = (rest == rest && fabsf(rest) != __builtin_inff()) ? f32_to_f16_sat(rest) : (uint16_t)0;
+    };
+    uint64_t i = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (i + 4 <= n && (n & 3u) == 0) {                 // (n a multiple of four keeps the second matrix 8-byte aligned)
+        const float4 v = *reinterpret_cast<const float4 *>(in + i);
+        uint16_t h[4], l[4];
+        one(v.x, h[0], l[0]); one(v.y, h[1], l[1]); one(v.z, h[2], l[2]); one(v.w, h[3], l[3]);
+        *reinterpret_cast<uint2 *>(out + i) = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+        *reinterpret_cast<uint2 *>(out + n + i) = make_uint2((uint32_t)l[0] | ((uint32_t)l[1] << 16), (uint32_t)l[2] | ((uint32_t)l[3] << 16));
+    } else {
+        for (uint64_t e = i; e < n && e < i + 4; ++e) one(in[e], out[e], out[n + e]);
+    }
 }
 
 // largest bit pattern of |w| among the finite BF16 values of an array
@@ -1353,7 +1361,7 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
     const void *in = d_x;
     if (split && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
-        sp_cvt16_split<<<(uint32_t)((cnt + 255) / 256), 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
+        sp_cvt16_split<<<(uint32_t)((cnt / 4 + 255) / 256 + 1), 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
         in = wk.buf[1];
     } else if (reg == R_GEMM16 && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];

@@ -44,6 +44,8 @@ CASES = [
     ("f16", [512, 768, 300], ["tanh", "none"], (300, 5), 0),
     ("f32", [784, 512, 1000, 10], ["relu", "relu", "softmax"], (256, 70), 0),      # FP32 matrix-core GEMM, split K
     ("f32", [96, 160, 10], ["foo52", "softmax"], (64, 1), 0),
+    ("i4", [256, 512, 384, 40], ["relu", "tanh", "softmax"], (300, 9), 128),       # split activations: partial sums of both matrices
+    ("bf16", [512, 1024, 1000], ["leaky_relu", "softmax"], (2048, 70), 128),
 ]
 
 
