@@ -28,7 +28,14 @@ __global__ __launch_bounds__(256) void sp_gemm32_f32(const Gemm32Args g)
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const uint32_t tiles_n = (N + BN - 1) / BN;
-    const uint32_t m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    // consecutive workgroups go to different XCDs: give each XCD a contiguous run of tiles, so that the tiles that
+    // share a row panel of A meet in one L2
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = gridDim.x / 8u;
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    const uint32_t m0 = (bid / tiles_n) * BM, n0 = (bid % tiles_n) * BN;
     const uint32_t kbeg = blockIdx.y * g.kper;
     const uint32_t kend = kbeg + g.kper < K ? kbeg + g.kper : K;
     const float *Wf = reinterpret_cast<const float *>(g.L.w);
