@@ -55,6 +55,10 @@ WORKLOADS = {
                init=["he"] * 5, prec=S.PRECISION_INT2, inputs="u11", batches=[1 << i for i in range(17)],
                # the batches whose dominant layer is also timed on its own (a roofline entry per row)
                roofline_batches=[1, 8, 64, 512, 4096, 65536]),
+    # not one of the reference's configurations: FP32 weights at a batch where the matrix cores decide, to show the
+    # FP32 matrix-core kernels next to the split mode (three FP16 products per layer)
+    "F1": dict(topo=[4096] * 4 + [1000], acts=["relu", "tanh", "relu", "softmax"], init=["he"] * 4,
+               prec=S.PRECISION_FLOAT32, inputs="n01", batches=[8192]),
 }
 
 
@@ -320,6 +324,15 @@ def run_workload(name, batches, steps, warmup, want_output=False, cpu_budget_s=0
             row["bf16_activations"] = dict(ms_per_step=w_wall, samples_per_s=n / (w_wall * 1e-3),
                                            mfma_frac=fl / (w_ev * 1e-3) / MFMA16_PEAK, dominant_layer_ms=w_layer,
                                            dominant_layer_frac=2.0 * n * topo[l - 1] * topo[l] / (w_layer * 1e-3) / MFMA16_PEAK)
+        if prec == S.PRECISION_FLOAT32 and n > 64 and (alternatives or name == "F1") and \
+                any(topo[l + 1] >= 128 and 2.0 * n * topo[l] * topo[l + 1] >= 3e9 for l in range(len(topo) - 1)):
+            # FP32 weights in split mode: every layer as three FP16 products into one FP32 accumulator (FP32-grade
+            # outputs); fractions are of the algorithmic flops against the FP32 matrix peak, which this mode may exceed
+            alt = S.SPHIP_SPLIT_ACTIVATIONS
+            w_wall, w_ev, y3 = time_workload(copies, topo, n, x, k, warmup, alt)
+            row["split_mode"] = dict(ms_per_step=w_wall, samples_per_s=n / (w_wall * 1e-3),
+                                     fp32_mfma_frac=fl / (w_ev * 1e-3) / FP32_PEAK,
+                                     max_abs_diff_to_fp32_kernels=float(np.max(np.abs(y3.astype(np.float64) - y))))
         if alternatives and want_output and prec != S.PRECISION_FLOAT32 and n >= 5:
             # the same workload with split activations (SPHIP_SPLIT_ACTIVATIONS / spingalett_set_net_activations): two
             # FP16 numbers per activation, twice the matrix-core work, FP32-grade outputs; the opt-in setting that
@@ -393,6 +406,8 @@ def compact_row(row):
         out["fwd_us"] = row["public_forward_us"]
     if "cpu_baseline_b1" in row:
         out["cpu_b1"] = row["cpu_baseline_b1"]
+    if "split_mode" in row:
+        out["split_mode"] = row["split_mode"]
     return out
 
 
@@ -560,7 +575,7 @@ def main():
 
     extra, cpu_extra, monotone = [], {}, {}
     if not args.no_extra:
-        for name in ("C2", "C3", "C5", "C1"):
+        for name in ("C2", "C3", "C5", "C1", "F1"):
             if name == args.workload:
                 continue
             try:
@@ -595,6 +610,7 @@ def main():
         "whole_net_mfma_frac": row["mfma_frac"], "whole_net_hbm_frac": row["hbm_frac"],
         "bf16_activations": row.get("bf16_activations"),
         "split_activations": row.get("split_activations"),
+        "split_mode": row.get("split_mode"),
         "cpu_baseline": cpu,
         # the other configurations, one short row per batch (keys: compact_row), their CPU legs once per configuration,
         # and whether samples/s is monotone in the batch up to 4096 samples (the GEMV -> GEMM crossover)

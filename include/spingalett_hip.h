@@ -58,7 +58,12 @@ typedef struct {
  * 22 significant bits together (the reference keeps FP32 activations, Training.c:313-345).  Each layer multiplies the
  * weights with both matrices (twice the matrix-core work) into FP32 partial sums that a second launch adds.  For nets
  * whose decisions hang on differences below FP16's 11 bits (many-class softmax heads); supersedes
- * SPHIP_BF16_ACTIVATIONS. */
+ * SPHIP_BF16_ACTIVATIONS.
+ * FP32 weights (beyond 64 samples): the weights are split the same way (made on the first such call, six more bytes
+ * per weight), and every layer runs as three FP16 products into one FP32 accumulator, hi x hi + lo x hi + hi x lo,
+ * instead of on the FP32 matrix instructions: about three times their throughput, outputs as close to the
+ * reference's as theirs (the dropped lo x lo term is 2^-22 of the sum).  Activations between the layers stay FP32;
+ * magnitudes beyond FP16's 65504 saturate in this mode, as in every 16-bit mode. */
 #define SPHIP_SPLIT_ACTIVATIONS 128u
 
 SPHIP_API int  sphip_device_count(void);
@@ -97,7 +102,8 @@ SPHIP_API int  sphip_forward(sphip_net *net, const float *x, uint32_t n, float *
  * Nothing in the array needs clearing between calls: every kernel reads only what this call wrote.  All calls on one
  * GPU share the array, so two calls that overlap in time (from different threads) race; nets of more than 64 layers
  * are refused.  flags: SPHIP_FORCE_GEMM / SPHIP_FORCE_GEMV / SPHIP_BF16_ACTIVATIONS /
- * SPHIP_SPLIT_ACTIVATIONS only. */
+ * SPHIP_SPLIT_ACTIVATIONS only (the latter on an FP32 net only after a sphip_forward with that flag has made the
+ * FP16 parts of the weights: making them allocates). */
 #define SPHIP_NOALLOC_SCRATCH_BYTES (64u << 20)
 SPHIP_API int  sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d_y, uint32_t flags);
 /* The evaluation step that follows batch_forward in the reference's epoch loop, on the device:

@@ -487,6 +487,86 @@ __global__ __launch_bounds__(256) void sp_bf16_to_f16(const uint16_t *__restrict
 #include "hip_gemm32.inl"
 
 // ---------------------------------------------------------------------------
+// FP32 weights on the 16-bit matrix cores (split mode of an FP32 net beyond 64 samples).  With FP16 parts
+// w 2^shift = wh + wl and x = xh + xl 2^-11,
+//     2^shift sum x w = sum xh wh + sum xl (wh 2^-11) + sum xh wl        (xl wl, 2^-22 of it, is dropped),
+// three FP16 products into one FP32 accumulator, i.e. one product over 3 Kp with the parts side by side along k:
+// activations [xh | xl | xh], weights [wh | wh 2^-11 | wl]; Kp = K rounded up to 8 elements, padded with zeros.
+// The shift brings the array's largest magnitude into [2^14, 2^15), so wl and wh 2^-11 keep their bits except for
+// weights 2^-12 of the largest and smaller, whose error is 2^-24 of the largest.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sp_cat3_x(const float *__restrict__ x, uint16_t *__restrict__ out, uint32_t n, uint32_t K,
+                                                 uint32_t Kp, int vec)
+{
+    const uint32_t groups = Kp / 8u;                      // one thread per 8 consecutive k of a row
+    const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (id >= (uint64_t)n * groups) return;
+    const uint32_t r = (uint32_t)(id / groups), k0 = (uint32_t)(id % groups) * 8u;
+    const float *src = x + (size_t)r * K + k0;
+    float v[8];
+    if (vec && k0 + 8u <= K) {
+        const float4 a = *reinterpret_cast<const float4 *>(src), b = *reinterpret_cast<const float4 *>(src + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = k0 + e < K ? src[e] : 0.0f;
+    }
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        uint16_t h0, l0, h1, l1;
+        split_f16(v[2 * e], h0, l0);
+        split_f16(v[2 * e + 1], h1, l1);
+        hi[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        lo[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+    }
+    uint16_t *row = out + (size_t)r * 3u * Kp + k0;
+    const uint4 H = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    *reinterpret_cast<uint4 *>(row) = H;
+    *reinterpret_cast<uint4 *>(row + Kp) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    *reinterpret_cast<uint4 *>(row + 2u * Kp) = H;
+}
+
+// largest bit pattern of |w| among the finite values of an FP32 array
+__global__ __launch_bounds__(256) void sp_absmax_f32(const float *__restrict__ w, uint64_t n, uint32_t *__restrict__ out)
+{
+    uint32_t m = 0;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256u) {
+        const uint32_t a = __float_as_uint(w[i]) & 0x7FFFFFFFu;
+        if (a < 0x7F800000u && a > m) m = a;
+    }
+    for (int off = 32; off; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)m, off);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
+}
+
+// one thread per weight: the three FP16 parts of w 2^shift, into the row's three sections; the padding is zeroed by
+// the threads of the row's last elements
+__global__ __launch_bounds__(256) void sp_cat3_w(const float *__restrict__ w, uint16_t *__restrict__ out, uint32_t N, uint32_t K,
+                                                 uint32_t Kp, int shift)
+{
+    const uint64_t id = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (id >= (uint64_t)N * Kp) return;
+    const uint32_t r = (uint32_t)(id / Kp), k = (uint32_t)(id % Kp);
+    uint16_t h = 0, hs = 0, l = 0;
+    if (k < K) {
+        const float v = ldexpf(w[(size_t)r * K + k], shift);
+        h = f32_to_f16_sat(v);
+        _Float16 hh;
+        __builtin_memcpy(&hh, &h, 2);
+        const float rest = v - (float)hh;                     // exact in FP32
+        l = (rest == rest && fabsf(rest) != __builtin_inff()) ? f32_to_f16_sat(rest) : (uint16_t)0;
+        hs = f32_to_f16_sat((float)hh * (1.0f / 2048.0f));
+    }
+    uint16_t *row = out + (size_t)r * 3u * Kp + k;
+    row[0] = h;
+    row[Kp] = hs;
+    row[2u * Kp] = l;
+}
+
+// ---------------------------------------------------------------------------
 // small copies (host staging of single-sample forwards)
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void sp_copy32(const float *__restrict__ src, float *__restrict__ dst, uint64_t n)
@@ -614,6 +694,9 @@ struct DevArray {
     uint16_t *wide16 = nullptr;    // BF16 weight arrays: the weights times 2^wide_shift as FP16 (made at upload)
     bool wide16_valid = false;
     int wide_shift = 0;
+    uint16_t *cat3 = nullptr;      // FP32 weight arrays in split mode: [out][3 Kp] FP16 parts of w 2^cat3_shift (made on demand)
+    bool cat3_valid = false;
+    int cat3_shift = 0;
 };
 
 struct sphip_train_state;
@@ -629,6 +712,7 @@ struct Workspace {
     float *split_ws;               // partial sums of K splits
     uint64_t split_cap;            // ... and how many floats it holds
     uint16_t *const *codes16;      // [layers-1]: FP16 copy of the codes of an integer layer with few outputs, or nullptr
+    uint16_t *cat;                 // split mode of an FP32 net: the three-part FP16 form of the current layer's input
 };
 
 struct sphip_net {
@@ -665,10 +749,12 @@ struct sphip_net {
     uint64_t eval_cap = 0;
     sphip_train_state *train = nullptr;   // gradients, optimizer moments, kept activations (training only)
     std::vector<uint16_t *> codes16_ptrs; // [layers-1] what Workspace::codes16 points at for the net's own workspace
+    uint16_t *cat_buf = nullptr;   // split mode of an FP32 net: three-part FP16 layer input
+    uint64_t cat_cap = 0;          // ... in elements
 
     Workspace workspace() const
     {
-        return Workspace{{buf[0], buf[1]}, aq, aq_inv, aq_dsum, soft_tmp, split_ws, split_cap, codes16_ptrs.data()};
+        return Workspace{{buf[0], buf[1]}, aq, aq_inv, aq_dsum, soft_tmp, split_ws, split_cap, codes16_ptrs.data(), cat_buf};
     }
 };
 
@@ -676,11 +762,14 @@ namespace {
 
 void train_free(sphip_net *net);
 
-enum Regime { R_GEMV, R_GEMM16, R_GEMM32 };
+// R_CAT3: FP32 weights, the larger layers as three FP16 products (cat3_layer, sp_cat3_x, sp_cat3_w), FP32 activations
+// between the layers
+enum Regime { R_GEMV, R_GEMM16, R_GEMM32, R_CAT3 };
 
 Regime pick_regime(const sphip_net *net, uint32_t n, uint32_t flags)
 {
     if ((flags & SPHIP_FORCE_GEMV) && n <= 64) return R_GEMV;
+    if (net->prec == F32 && (flags & SPHIP_SPLIT_ACTIVATIONS) && n > 64) return R_CAT3;
     if (flags & SPHIP_FORCE_GEMM) return net->prec == F32 ? R_GEMM32 : R_GEMM16;
     if (net->prec == F32) return n <= 64 ? R_GEMV : R_GEMM32;
     return n <= 4 ? R_GEMV : R_GEMM16;
@@ -1225,6 +1314,7 @@ struct WorkspaceNeed {
     uint64_t plane_bytes;      // digit planes: 4 bytes per element (+ padding of the last chunk) ...
     uint64_t plane_recs;       // ... and one scale (+ four digit sums) per 64 elements
     uint64_t split_floats;
+    uint64_t cat_elems;        // split mode of an FP32 net: FP16 elements of the widest three-part layer input
 };
 
 // an integer layer with at most 64 outputs streams the activations against an FP16 copy of its codes
@@ -1235,11 +1325,21 @@ bool layer_wants_codes16(const sphip_net *net, uint32_t l /*1-based*/, uint32_t 
     return tp.use && tp.mode_b;
 }
 
-// halves = 2: a split-activation forward, in which every matrix-core layer writes one set of partial sums per
-// activation matrix
-WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t halves = 1)
+uint32_t cat3_kp(uint32_t K) { return (K + 7u) & ~7u; }
+
+// Split mode of an FP32 net: which layers run as three FP16 products.  Measured against sp_gemm32_f32 on layers of
+// 512 to 4096 inputs and outputs, conversion of the input included: even at 1-2 GFLOP per layer, 1.4x at 4 GFLOP,
+// 2.6x at 70 GFLOP; layers of a hundred outputs and fewer lose at every batch tried (streaming kernels over a row
+// three times as long).  The other layers keep the FP32 kernel; FP32 activations between the layers either way.
+bool cat3_layer(uint32_t n, uint32_t N, uint32_t K) { return N >= 128u && 2.0 * (double)n * N * K >= 3e9; }
+
+// In a split-activation forward of a 16-bit or integer net every matrix-core layer writes one set of partial sums per
+// activation matrix (halves = 2)
+WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t flags)
 {
     WorkspaceNeed w{};
+    const Regime reg = pick_regime(net, n, flags);
+    const uint32_t halves = (flags & SPHIP_SPLIT_ACTIVATIONS) && reg == R_GEMM16 ? 2u : 1u;
     w.act_floats = (uint64_t)n * net->max_width;
     for (uint32_t l = 1; l < net->layers; ++l)
         if (net->act[l - 1] == A_SOFTMAX && (uint64_t)n * net->topo[l] > w.soft_floats) w.soft_floats = (uint64_t)n * net->topo[l];
@@ -1252,7 +1352,17 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t halves =
         const uint32_t N = net->topo[l], K = net->topo[l - 1];
         uint32_t kper = 0;
         uint64_t ws = 0;
-        if (net->prec == F32) {
+        if (reg == R_CAT3 && cat3_layer(n, N, K)) {
+            const uint32_t K3 = 3u * cat3_kp(K);
+            if ((uint64_t)n * K3 > w.cat_elems) w.cat_elems = (uint64_t)n * K3;
+            const ThinPlan tp = plan_thin(F16, n, N, K3);
+            if (tp.use) {
+                if (tp.splits > 1) ws = (uint64_t)tp.splits * tp.NC * tp.R;
+            } else {
+                const uint32_t sp = gemm16_splits(F16, n, N, K3, &kper);
+                if (sp > 1) ws = (uint64_t)sp * n * N;
+            }
+        } else if (net->prec == F32) {
             if (n <= 64) continue;
             const uint32_t sp = gemm32_splits(n, N, K, &kper);
             if (sp > 1) ws = (uint64_t)sp * n * N;
@@ -1278,10 +1388,43 @@ void launch_codes16(int prec, const uint8_t *codes, uint16_t *out, uint64_t coun
     else sp_codes16<I2><<<grid, 256, 0, g_stream>>>(codes, out, count);
 }
 
-// grows the net's own workspace to what n samples need
-int reserve(sphip_net *net, uint32_t n, bool keep_layers, uint32_t halves = 1)
+// The three-part FP16 form of an FP32 weight array [N][K] (sp_cat3_w): one small reduction for the shift, one wait,
+// one conversion.  The word the reduction leaves its result in sits behind the copy, in the same allocation.
+int make_cat3(DevArray &wa, uint32_t N, uint32_t K)
 {
-    const WorkspaceNeed need = workspace_need(net, n, halves);
+    const uint32_t Kp = cat3_kp(K);
+    const size_t copy_bytes = (size_t)N * 3u * Kp * sizeof(uint16_t);          // a multiple of 16
+    if (!wa.cat3) HCHECK(hipMalloc((void **)&wa.cat3, copy_bytes + 16u));
+    uint32_t *word = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(wa.cat3) + copy_bytes);
+    const float *src = reinterpret_cast<const float *>(wa.base);
+    uint32_t top = 0;
+    HCHECK(hipMemsetAsync(word, 0, sizeof(uint32_t), g_stream));
+    uint64_t blocks = (wa.count + 255) / 256;
+    if (blocks > 512) blocks = 512;                       // (every wave ends in one atomic on the same word)
+    sp_absmax_f32<<<(uint32_t)blocks, 256, 0, g_stream>>>(src, wa.count, word);
+    HCHECK(hipMemcpyAsync(&top, word, sizeof(uint32_t), hipMemcpyDeviceToHost, g_stream));
+    HCHECK(hipStreamSynchronize(g_stream));
+    wa.cat3_shift = top ? 14 - ((int)(top >> 23) - 127) : 0;       // largest magnitude = 1.m x 2^(e - 127)
+    sp_cat3_w<<<(uint32_t)(((uint64_t)N * Kp + 255) / 256), 256, 0, g_stream>>>(src, wa.cat3, N, K, Kp, wa.cat3_shift);
+    HCHECK(hipGetLastError());
+    wa.cat3_valid = true;
+    return 0;
+}
+
+// grows the net's own workspace to what n samples need
+int reserve(sphip_net *net, uint32_t n, bool keep_layers, uint32_t flags = 0)
+{
+    const WorkspaceNeed need = workspace_need(net, n, flags);
+    if (need.cat_elems > net->cat_cap) {
+        if (net->cat_buf) { HCHECK(hipFree(net->cat_buf)); net->cat_buf = nullptr; }
+        net->cat_cap = 0;
+        HCHECK(hipMalloc((void **)&net->cat_buf, need.cat_elems * sizeof(uint16_t)));
+        net->cat_cap = need.cat_elems;
+    }
+    if (need.cat_elems)
+        for (uint32_t l = 1; l < net->layers; ++l)
+            if (cat3_layer(n, net->topo[l], net->topo[l - 1]) && !net->W[l - 1].cat3_valid && net->W[l - 1].uploaded &&
+                make_cat3(net->W[l - 1], net->topo[l], net->topo[l - 1])) return 1;
     if (need.act_floats > net->cap_elems) {
         for (int i = 0; i < 2; ++i) {
             if (net->buf[i]) { HCHECK(hipFree(net->buf[i])); net->buf[i] = nullptr; }
@@ -1379,6 +1522,13 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
             L.w = reinterpret_cast<const uint8_t *>(net->W[l - 1].wide16);
             L.wscale = ldexpf(L.wscale, -net->W[l - 1].wide_shift);
         }
+        const bool cat3 = reg == R_CAT3 && cat3_layer(n, L.N, L.K);
+        if (cat3) {
+            if (!net->W[l - 1].cat3_valid) return fail_msg("sphip: the FP16 parts of this net's FP32 weights were not made (split mode)");
+            L.w = reinterpret_cast<const uint8_t *>(net->W[l - 1].cat3);
+            L.wscale = ldexpf(L.wscale, -net->W[l - 1].cat3_shift);
+            L.K = 3u * cat3_kp(net->topo[l - 1]);
+        }
         const bool softmax = net->act[l - 1] == A_SOFTMAX;
         const bool is_last = l == last;
         void *dst = is_last ? (void *)d_y : keep ? (void *)(net->layers_buf + net->slot_off[l]) : wk.buf[(l + 1) & 1];
@@ -1390,10 +1540,25 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
         if (run) {
             if (reg == R_GEMV) launch_gemv(net->prec, wk, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
-            else if (reg == R_GEMM32)
+            else if (reg == R_GEMM32 || (reg == R_CAT3 && !cat3))
                 soft_done = launch_gemm32(L, (const float *)in, (float *)main_out, n, wk.split_ws, wk.split_cap,
                                           softmax && !only_layer ? (float *)dst : nullptr);
-            else {
+            else if (cat3) {
+                // (timing one layer includes the conversion of its input)
+                const uint32_t K = net->topo[l - 1], Kp = cat3_kp(K);
+                const int vec = K % 4u == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+                sp_cat3_x<<<(uint32_t)(((uint64_t)n * (Kp / 8u) + 255) / 256), 256, 0, g_stream>>>((const float *)in, wk.cat, n, K, Kp, vec);
+                ThinCtx ctx{};
+                ctx.w16 = net->W[l - 1].cat3;
+                ctx.ws = wk.split_ws;
+                ctx.ws_floats = wk.split_cap;
+                if (softmax && !only_layer) {
+                    ctx.soft_out = dst;
+                    ctx.soft_kind = 0;
+                    ctx.soft_done = &soft_done;
+                }
+                launch_gemm16((int)F16, L, wk.cat, main_out, n, 1, ctx);
+            } else {
                 const DevArray &wa = net->W[l - 1];
                 ThinCtx ctx{};
                 if (wide) ctx.w16 = wa.wide16;
@@ -1446,9 +1611,8 @@ uint32_t batch_block_rows(const sphip_net *net, uint32_t n, uint32_t flags)
 int reserve_batch(sphip_net *net, uint32_t n, uint32_t flags)
 {
     const uint32_t rows = batch_block_rows(net, n, flags);
-    const uint32_t halves = (flags & SPHIP_SPLIT_ACTIVATIONS) ? 2u : 1u;
-    if (reserve(net, rows, false, halves)) return 1;
-    if (rows < n && n % rows != 0 && reserve(net, n % rows, false, halves)) return 1;
+    if (reserve(net, rows, false, flags)) return 1;
+    if (rows < n && n % rows != 0 && reserve(net, n % rows, false, flags)) return 1;
     return 0;
 }
 
@@ -1522,9 +1686,10 @@ void sphip_destroy(sphip_net *net)
     if (!net) return;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
     train_free(net);
-    for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); if (a.wide16) (void)hipFree(a.wide16); }
+    for (auto &a : net->W) { if (a.base) (void)hipFree(a.base); if (a.codes16) (void)hipFree(a.codes16); if (a.wide16) (void)hipFree(a.wide16); if (a.cat3) (void)hipFree(a.cat3); }
     for (auto &a : net->B) if (a.base) (void)hipFree(a.base);
     if (net->split_ws) (void)hipFree(net->split_ws);
+    if (net->cat_buf) (void)hipFree(net->cat_buf);
     if (net->eval_buf) (void)hipFree(net->eval_buf);
     for (int i = 0; i < 2; ++i) if (net->buf[i]) (void)hipFree(net->buf[i]);
     if (net->soft_tmp) (void)hipFree(net->soft_tmp);
@@ -1575,6 +1740,7 @@ int sphip_upload_array(sphip_net *net, uint32_t l, int which, const void *codes,
     a.uploaded = true;
     a.codes16_valid = false;
     a.wide16_valid = false;
+    a.cat3_valid = false;
     if (which == 0 && net->prec == BF16 && make_wide(a)) return 1;
     return 0;
 }
@@ -1763,7 +1929,11 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
         if (scratch_lookup(&base)) return 1;
     }
     // lay the workspace out inside the scratch array, every piece at a multiple of 256 bytes
-    const WorkspaceNeed need = workspace_need(net, n, (flags & SPHIP_SPLIT_ACTIVATIONS) ? 2u : 1u);
+    const WorkspaceNeed need = workspace_need(net, n, flags);
+    if (need.cat_elems)
+        for (uint32_t l = 1; l < net->layers; ++l)
+            if (cat3_layer(n, net->topo[l], net->topo[l - 1]) && !net->W[l - 1].cat3_valid)
+                return fail_msg("sphip_forward_noalloc: the split mode of an FP32 net needs FP16 parts of its weights, which the first sphip_forward in that mode makes");
     size_t used = 0;
     auto take = [&](uint64_t bytes) -> unsigned char * {
         unsigned char *p = base + used;
@@ -1782,6 +1952,7 @@ int sphip_forward_noalloc(sphip_net *net, const float *d_x, uint32_t n, float *d
     }
     wk.split_ws = reinterpret_cast<float *>(take(need.split_floats * sizeof(float)));
     wk.split_cap = need.split_floats;
+    if (need.cat_elems) wk.cat = reinterpret_cast<uint16_t *>(take(need.cat_elems * sizeof(uint16_t)));
     // an integer layer with few outputs reads an FP16 copy of its codes: the net's own if an earlier call made one,
     // else one made here, in the scratch array, on every call
     // (only the matrix-core regime reads them: a forced vector forward or one of up to four samples never does)
@@ -2036,6 +2207,19 @@ const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, 
     case R_GEMM32:
         (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
         break;
+    case R_CAT3: {
+        if (!cat3_layer(n, L.N, L.K)) {
+            (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
+            break;
+        }
+        LayerArgs L3 = L;
+        L3.K = 3u * cat3_kp(L.K);
+        ThinCtx ctx{};
+        ctx.w16 = reinterpret_cast<const uint16_t *>(aligned_ptr);
+        ctx.ws_floats = ~0ull;
+        launch_gemm16((int)F16, L3, reinterpret_cast<const uint16_t *>(aligned_ptr), nullptr, n, 1, ctx);
+        break;
+    }
     default: {
         ThinCtx ctx{};
         ctx.w16 = reinterpret_cast<const uint16_t *>(aligned_ptr);

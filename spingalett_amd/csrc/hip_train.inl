@@ -494,6 +494,7 @@ int sphip_train_set(sphip_net *net, int which, uint32_t l, const float *host)
     if (!dst) return fail_msg("sphip_train_set: unknown array");
     HCHECK(hipMemcpyAsync(dst, host, cnt * sizeof(float), hipMemcpyHostToDevice, g_stream));
     HCHECK(hipStreamSynchronize(g_stream));
+    if (which == SPHIP_TRAIN_W) net->W[l].cat3_valid = false;      // the FP16 parts describe the old weights
     return 0;
 }
 
@@ -605,6 +606,7 @@ int sphip_train_step(sphip_net *net, const float *x, const float *targets, uint3
         const uint64_t wc = (uint64_t)net->topo[l] * net->topo[l + 1], bc = net->topo[l + 1];
         launch_opt(*args, reinterpret_cast<float *>(net->W[l].base), ts->gW + ts->woff[l], ts->mW + ts->woff[l], ts->vW + ts->woff[l],
                    wc, args->weight_decay, clip);
+        net->W[l].cat3_valid = false;                               // the FP16 parts of a split-mode forward describe the old weights
         launch_opt(*args, reinterpret_cast<float *>(net->B[l].base), ts->gB + ts->boff[l], ts->mB + ts->boff[l], ts->vB + ts->boff[l],
                    bc, 0.0f, clip);
     }

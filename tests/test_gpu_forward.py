@@ -424,6 +424,78 @@ def test_split_activations_on_every_kernel_family(S, O, fmt, topo, acts, n):
     assert rel_max_abs(plain, want) <= TOL_MFMA
 
 
+# The split mode of an FP32 net: beyond 64 samples every layer of 128 outputs and more and at least 3 GFLOP runs as
+# three FP16 products into one FP32 accumulator (weights and activations as two FP16 parts each) instead of on the
+# FP32 matrix instructions; the other layers keep the FP32 kernel.
+_F32_SPLIT_CASES = [
+    # topology, activations, samples, inputs, input scale, which layers run on the 16-bit matrix cores
+    ([784, 512, 1000, 10], ["relu", "relu", "softmax"], 256, "u01", 1.0, (0, 0, 0)),    # configuration 1: too small
+    ([784, 512, 1000, 10], ["relu", "relu", "softmax"], 4096, "u01", 1.0, (1, 1, 0)),
+    ([1001, 515, 130], ["leaky_relu", "foo52"], 4100, "n01", 1.0, (1, 0)),     # rows that are not whole 16-byte units
+    ([2048, 384, 520, 33], ["sigmoid", "softmax", "none"], 3000, "n01", 1.0, (1, 0, 0)),   # hidden softmax behind it
+    ([1024, 2048, 1024, 1000], ["tanh", "leaky_relu", "softmax"], 2048, "n01", 1.0, (1, 1, 1)),   # K of 3 x 2048, softmax head
+    ([512, 768, 256], ["relu", "none"], 4096, "n01", 3e3, (1, 0)),           # large activations (up to about 1e5 x 0.03)
+    ([512, 768, 768], ["relu", "none"], 4096, "n01", 1e-4, (1, 1)),          # small ones: the low parts are FP16 subnormals
+]
+
+
+@pytest.mark.parametrize("topo,acts,n,inp,scale,on16", _F32_SPLIT_CASES)
+def test_split_mode_of_an_fp32_net_runs_on_the_16_bit_matrix_cores(S, O, topo, acts, n, inp, scale, on16):
+    """FP32 weights, split mode, more than 64 samples: the outputs stay within the FP32 bar (1e-4 of the float64
+    forward; measured about 1e-6, as close as the FP32 matrix-core path) while the large layers run in a 16-bit kernel
+    over three times the padded row length."""
+    src = make_oracle_net(O, topo, acts, seed=n + len(topo), bias_std=0.1)
+    _, ref, net = quantized_pair(O, S, src, "f32")
+    rng = np.random.default_rng(n)
+    X = (rng.random((n, topo[0]), dtype=F32) if inp == "u01" else rng.standard_normal((n, topo[0])).astype(F32)) * F32(scale)
+    want = ref.forward_batch_f64(X)
+    plain = S.forward_batch(net, X)
+    assert S.lib().spingalett_set_net_activations(net, S.NET_ACTIVATIONS_SPLIT) == 0
+    got = S.forward_batch(net, X)
+    m = n * 7 // 8                                                 # a smaller batch through the same buffers
+    again = S.forward_batch(net, X[:m])
+    h = S.lib().spingalett_hip_handle(net)
+    names = [S.lib().sphip_layer_kernel_name(h, l, n, S.SPHIP_SPLIT_ACTIVATIONS).decode() for l in range(1, len(topo))]
+    few = S.forward_batch(net, X[:64])                             # up to 64 samples stay on the FP32 vector kernels
+    S.free_network(net)
+    assert rel_max_abs(plain, want) <= TOL_VEC
+    assert rel_max_abs(got, want) <= 2e-5, (topo, n, rel_max_abs(got, want), rel_max_abs(plain, want))
+    assert rel_max_abs(again, want[:m]) <= 2e-5
+    assert rel_max_abs(few, want[:64]) <= TOL_VEC
+    assert [k.startswith(("sp_gemm16", "sp_skinny16")) for k in names] == [bool(x) for x in on16], names
+    assert all(k == "sp_gemm32_f32" for k, x in zip(names, on16) if not x), names
+    if not any(on16):
+        assert np.array_equal(got, plain)
+
+
+def test_split_mode_of_an_fp32_net_follows_new_weights(S, O):
+    """The FP16 parts of the weights are made on demand and made again after the arrays change on the device: by an
+    upload, and by a training step."""
+    topo, acts, n = [640, 768, 8], ["tanh", "none"], 3200               # first layer 3.1 GFLOP: on the 16-bit matrix cores
+    a = make_oracle_net(O, topo, acts, seed=1)
+    b = make_oracle_net(O, topo, acts, seed=2)
+    X = np.random.default_rng(0).standard_normal((n, topo[0])).astype(F32)
+    d = S.DeviceNet(topo, [S.ACT_TANH, S.ACT_NONE], S.PRECISION_FLOAT32)
+    for src in (a, b):
+        for l in range(2):
+            d.upload(l, 0, np.ascontiguousarray(src.W(l)).ravel())
+            d.upload(l, 1, np.ascontiguousarray(src.b(l)).ravel())
+        got = d.forward(X, S.SPHIP_SPLIT_ACTIVATIONS)
+        assert rel_max_abs(got, src.forward_batch_f64(X)) <= 2e-5
+    d.train_begin()
+    args = S.SphipTrainArgs(S.OPTIMIZER_SGD, S.LOSS_MSE, 0.05, 0.0, 0.9, 0.9, 0.999, 1e-8, 0.0, 0.9, 0.999)
+    T = np.random.default_rng(1).standard_normal((n, topo[-1])).astype(F32)
+    d.train_step(X, T, args)
+    trained = O.Net.new(topo, [O.ACT[x] for x in acts], 0)
+    for l in range(2):
+        trained.W(l)[:] = d.train_get(S.SPHIP_TRAIN_W, l).reshape(trained.W(l).shape)
+        trained.b(l)[:] = d.train_get(S.SPHIP_TRAIN_B, l)
+    got = d.forward(X, S.SPHIP_SPLIT_ACTIVATIONS)
+    assert rel_max_abs(got, trained.forward_batch_f64(X)) <= 2e-5
+    assert rel_max_abs(got, b.forward_batch_f64(X)) > 1e-3              # the step moved the outputs
+    d.destroy()
+
+
 def test_net_activation_mode_arguments(S, O):
     src = make_oracle_net(O, [8, 4], ["none"], seed=1)
     _, ref, net = quantized_pair(O, S, src, "i8")

@@ -79,6 +79,30 @@ def test_noalloc_forward_equals_forward(S, fmt, topo, acts, ns, flags):
     fresh.destroy()
 
 
+def test_noalloc_forward_in_the_split_mode_of_an_fp32_net(S):
+    """That mode reads FP16 parts of the weights, which are made (allocated) by the first sphip_forward in the mode:
+    before it the entry point refuses, after it the call works out of the scratch array like every other route."""
+    topo, n = [1024, 2048, 10], 768                       # first layer 3.2 GFLOP: three FP16 products; the head: FP32 kernel
+    net = _net(S, "f32", topo, [S.ACT_RELU, S.ACT_SOFTMAX], seed=3)
+    X = np.random.default_rng(4).random((n, topo[0]), dtype=F32)
+    d_x = S.DeviceBuffer.from_numpy(X)
+    d_y = S.DeviceBuffer(n * topo[-1] * 4)
+    assert net.forward_noalloc(d_x, n, d_y, S.SPHIP_SPLIT_ACTIVATIONS) == 1
+    assert "FP16 parts" in S.lib().sphip_last_error_string().decode()
+    want = net.forward(X, S.SPHIP_SPLIT_ACTIVATIONS)
+    for m in (n, 740):
+        assert net.forward_noalloc(d_x, m, d_y, S.SPHIP_SPLIT_ACTIVATIONS) == 0, S.lib().sphip_last_error_string()
+        S.synchronize()
+        free_before, _ = S.device_memory()
+        assert net.forward_noalloc(d_x, m, d_y, S.SPHIP_SPLIT_ACTIVATIONS) == 0
+        S.synchronize()
+        free_after, _ = S.device_memory()
+        assert free_after == free_before
+        ref = want[:m] if m == n else net.forward(X[:m], S.SPHIP_SPLIT_ACTIVATIONS)
+        assert np.array_equal(d_y.to_numpy(F32, (n, topo[-1]))[:m].view(np.uint32), ref.view(np.uint32)), m
+    net.destroy()
+
+
 def test_noalloc_forward_refuses_what_does_not_fit(S):
     """64 MiB of scratch: 8192 samples of a 4096-wide net need two 128 MiB activation buffers."""
     net = _net(S, "bf16", [256, 4096, 16], [S.ACT_RELU, S.ACT_NONE], seed=5)
