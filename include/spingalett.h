@@ -282,7 +282,7 @@ SPINGALETT_API SpingalettBf16Activations spingalett_get_bf16_activations(void);
  * value rounded to FP16, and the rounding error times 2^11: about 22 significant bits together) at twice the
  * matrix-core work per layer, for nets whose decisions hang on differences smaller than FP16's 11 bits — a softmax
  * over a thousand classes agrees with the reference's FP32 argmax on 99.9 % of random samples only this way.  For a
- * net with FP32 weights SPLIT is the fast setting for batches of more than 64 samples: weights and activations are
+ * net with FP32 weights SPLIT is the fast setting for large batches: weights and activations are
  * both taken as two FP16 numbers and every layer runs as three FP16 matrix-core products into one FP32 sum, about
  * three times the throughput of the FP32 matrix instructions at the same distance from the reference's outputs
  * (activations beyond FP16's 65504 saturate; six more bytes per weight on the device).  DEFAULT follows the

@@ -59,7 +59,7 @@ typedef struct {
  * weights with both matrices (twice the matrix-core work) into FP32 partial sums that a second launch adds.  For nets
  * whose decisions hang on differences below FP16's 11 bits (many-class softmax heads); supersedes
  * SPHIP_BF16_ACTIVATIONS.
- * FP32 weights (beyond 64 samples): the weights are split the same way (made on the first such call, six more bytes
+ * FP32 weights (five samples and more): the weights are split the same way (made on the first such call, six more bytes
  * per weight), and every layer runs as three FP16 products into one FP32 accumulator, hi x hi + lo x hi + hi x lo,
  * instead of on the FP32 matrix instructions: about three times their throughput, outputs as close to the
  * reference's as theirs (the dropped lo x lo term is 2^-22 of the sum).  Activations between the layers stay FP32;

@@ -766,12 +766,18 @@ void train_free(sphip_net *net);
 // between the layers
 enum Regime { R_GEMV, R_GEMM16, R_GEMM32, R_CAT3 };
 
+// FP32 weights: the vector kernel up to four samples, like every other format; beyond that the FP32 matrix-core kernel
+// with its K splits is the faster one, although the vector kernel takes eight samples per pass over the weights
+// (784-512-1000-10 at 5 / 8 / 64 samples: 27 / 34 / 245 us against 27 / 30 / 31 us; three 4096-wide layers 97 / 124 / 960
+// against 84 / 84 / 83 us; at four samples 16 against 29 and 42 against 85 us).
+constexpr uint32_t kF32VectorMax = 4;
+
 Regime pick_regime(const sphip_net *net, uint32_t n, uint32_t flags)
 {
     if ((flags & SPHIP_FORCE_GEMV) && n <= 64) return R_GEMV;
-    if (net->prec == F32 && (flags & SPHIP_SPLIT_ACTIVATIONS) && n > 64) return R_CAT3;
+    if (net->prec == F32 && (flags & SPHIP_SPLIT_ACTIVATIONS) && n > kF32VectorMax) return R_CAT3;
     if (flags & SPHIP_FORCE_GEMM) return net->prec == F32 ? R_GEMM32 : R_GEMM16;
-    if (net->prec == F32) return n <= 64 ? R_GEMV : R_GEMM32;
+    if (net->prec == F32) return n <= kF32VectorMax ? R_GEMV : R_GEMM32;
     return n <= 4 ? R_GEMV : R_GEMM16;
 }
 
@@ -1363,7 +1369,7 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t flags)
                 if (sp > 1) ws = (uint64_t)sp * n * N;
             }
         } else if (net->prec == F32) {
-            if (n <= 64) continue;
+            if (reg == R_GEMV) continue;
             const uint32_t sp = gemm32_splits(n, N, K, &kper);
             if (sp > 1) ws = (uint64_t)sp * n * N;
         } else {

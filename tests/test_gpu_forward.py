@@ -456,7 +456,7 @@ def test_split_mode_of_an_fp32_net_runs_on_the_16_bit_matrix_cores(S, O, topo, a
     again = S.forward_batch(net, X[:m])
     h = S.lib().spingalett_hip_handle(net)
     names = [S.lib().sphip_layer_kernel_name(h, l, n, S.SPHIP_SPLIT_ACTIVATIONS).decode() for l in range(1, len(topo))]
-    few = S.forward_batch(net, X[:64])                             # up to 64 samples stay on the FP32 vector kernels
+    few = S.forward_batch(net, X[:64])                             # too little work for the 16-bit route in every case here
     S.free_network(net)
     assert rel_max_abs(plain, want) <= TOL_VEC
     assert rel_max_abs(got, want) <= 2e-5, (topo, n, rel_max_abs(got, want), rel_max_abs(plain, want))
@@ -494,6 +494,23 @@ def test_split_mode_of_an_fp32_net_follows_new_weights(S, O):
     assert rel_max_abs(got, trained.forward_batch_f64(X)) <= 2e-5
     assert rel_max_abs(got, b.forward_batch_f64(X)) > 1e-3              # the step moved the outputs
     d.destroy()
+
+
+def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
+    """From five samples on the FP32 matrix-core kernel is the faster one for FP32 weights, as the 16-bit one is for
+    the other formats (configuration 1 at 64 samples: 31 us against 245 us in eight passes of the vector kernel), and
+    its K splits need their workspace at those batch sizes too."""
+    topo, acts = [784, 512, 1000, 10], ["relu", "relu", "softmax"]
+    src = make_oracle_net(O, topo, acts, seed=5, bias_std=0.1)
+    _, ref, net = quantized_pair(O, S, src, "f32")
+    h = S.lib().spingalett_hip_handle(net)
+    assert [S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() for n in (1, 4, 5, 64, 65)] == \
+        ["sp_gemv", "sp_gemv", "sp_gemm32_f32", "sp_gemm32_f32", "sp_gemm32_f32"]
+    X = np.random.default_rng(3).random((64, topo[0]), dtype=F32)
+    want = ref.forward_batch_f64(X)
+    for n in (4, 5, 9, 33, 64):
+        assert rel_max_abs(S.forward_batch(net, X[:n]), want[:n]) <= TOL_VEC, n
+    S.free_network(net)
 
 
 def test_net_activation_mode_arguments(S, O):
