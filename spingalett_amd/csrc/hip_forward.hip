@@ -998,6 +998,22 @@ uint32_t gemm16_splits(int fmt, uint32_t M, uint32_t N, uint32_t K, uint32_t *kp
     return (ktiles + per - 1) / per;
 }
 
+// K splits of the single-stage kernel for rows that are not whole 16-byte units (always 64 x 64 tiles, element-wise
+// loads): few samples give it a handful of workgroups, each walking all of K with nothing in flight (1030 x 777 at
+// 64 samples: 17 workgroups, 80 us).  Whole K tiles per split, about two workgroups per compute unit.
+uint32_t gemm16_ragged_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
+{
+    const uint32_t tiles = ((M + 63u) / 64u) * ((N + 63u) / 64u), ktiles = (K + 63u) / 64u;
+    *kper = 0;
+    if (tiles >= 256u || ktiles < 2u) return 1;
+    uint32_t splits = (512u + tiles - 1) / tiles;
+    if (splits > 16u) splits = 16u;
+    if (splits > ktiles) splits = ktiles;
+    const uint32_t per = (ktiles + splits - 1) / splits;
+    *kper = per * 64u;
+    return (ktiles + per - 1) / per;
+}
+
 // What the thin-operand kernel needs beyond the layer itself
 struct ThinCtx {
     const uint16_t *w16;   // [N][K] 16-bit weights (raw 16-bit formats, or FP16 codes) when N <= 64, else nullptr
@@ -1231,6 +1247,16 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     g.kper = 0;
     g.ksplits = 1;
     if (halves == 2) g.ws = ctx.ws;                  // one partial sum per activation matrix, added by the reduction
+    const bool words = !aligned && L.K % 8u == 0 && ((uint64_t)L.K * fmt_bits(FMT)) % 32u == 0 && (FMT == I8 || FMT == I4 || FMT == I2);
+    if (!aligned && !words) {
+        uint32_t kper = 0;
+        const uint32_t sp = gemm16_ragged_splits(M, L.N, L.K, &kper);
+        if (sp > 1 && (uint64_t)sp * halves * M * L.N <= ctx.ws_floats) {
+            g.kper = kper;
+            g.ksplits = sp;
+            g.ws = ctx.ws;
+        }
+    }
     tl_route.name = "sp_gemm16";
     if (tl_route.dry) return;
     // This kernel has one LDS stage, so it lives on the number of resident workgroups: the largest of 128 x 128,
@@ -1238,12 +1264,11 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     // 21.7 / 16.2 / 12.9 us, 8192 x 8192 x 1000 BF16 0.27 / 0.37 / 0.42 ms); the element-wise loads of unaligned
     // rows always want the smallest (8192 x 8192 x 1000 INT8: 1.90 / 1.69 / 1.51 ms).
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((L.N + bn - 1) / bn); };
-    // integer codes whose rows are whole 32-bit words (not whole 16-byte units) next to aligned activations
-    const bool words = !aligned && L.K % 8u == 0 && ((uint64_t)L.K * fmt_bits(FMT)) % 32u == 0 && (FMT == I8 || FMT == I4 || FMT == I2);
+    // (words: integer codes whose rows are whole 32-bit words, not whole 16-byte units, next to aligned activations)
     const int shape = !(aligned || words) ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
     auto go = [&](auto tm_c, auto tn_c) {
         constexpr int TM = decltype(tm_c)::value, TN = decltype(tn_c)::value;
-        const dim3 grid(tiles(64 * TM, 64 * TN), halves);
+        const dim3 grid(tiles(64 * TM, 64 * TN), g.ksplits * halves);
         if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
             if (words) {
                 sp_gemm16<FMT, F16T, TM, TN, true, true><<<grid, 256, 0, g_stream>>>(g);
@@ -1261,8 +1286,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     if (g.ws) {
         const uint64_t total = (uint64_t)M * L.N;
         const bool vec = L.N % 4u == 0 && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
-        if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, 1u);
-        else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, 1u);
+        if (vec) sp_gemm16_reduce<F16T, true><<<(uint32_t)((total / 4u + 255) / 256), 256, 0, g_stream>>>(g, g.ksplits);
+        else sp_gemm16_reduce<F16T, false><<<(uint32_t)((total + 255) / 256), 256, 0, g_stream>>>(g, g.ksplits);
     }
 }
 
@@ -1379,6 +1404,12 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t flags)
             } else {
                 const uint32_t sp = gemm16_splits(net->prec, n, N, K, &kper);
                 if (sp > 1 || halves > 1) ws = (uint64_t)sp * halves * n * N;
+                const bool aligned = rows_aligned(net->prec, K) && K % 8u == 0;
+                const bool words = !aligned && K % 8u == 0 && ((uint64_t)K * fmt_bits(net->prec)) % 32u == 0 && net->prec >= I8;
+                if (!aligned && !words) {
+                    const uint32_t rs = gemm16_ragged_splits(n, N, K, &kper);
+                    if (rs > 1) ws = (uint64_t)rs * halves * n * N;
+                }
             }
         }
         if (ws > w.split_floats) w.split_floats = ws;

@@ -140,7 +140,10 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     const uint32_t M = g.M, N = g.L.N, K = g.L.K;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const uint16_t *const A = g.A + (size_t)blockIdx.y * M * K;      // grid y > 1: the matrices of a split activation
+    // grid y = halves x K splits: y / ksplits picks the matrix of a split activation, y % ksplits the K range (whole tiles)
+    const uint16_t *const A = g.A + (size_t)(blockIdx.y / g.ksplits) * M * K;
+    const uint32_t kbeg = g.kper ? (blockIdx.y % g.ksplits) * g.kper : 0u;
+    const uint32_t kend = g.kper && kbeg + g.kper < K ? kbeg + g.kper : K;
 
     // tile index: consecutive workgroups go to different XCDs, so give each XCD a
     // contiguous band of tiles (shared A rows / W rows stay in one L2)
@@ -271,13 +274,13 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
         }
     };
 
-    const uint32_t ktiles = (K + BK - 1) / BK;
-    load_tiles(0);
+    const uint32_t ktiles = (kend - kbeg + BK - 1) / BK;
+    load_tiles(kbeg);
     for (uint32_t kt = 0; kt < ktiles; ++kt) {
         __syncthreads();                              // previous tile fully consumed
-        store_tiles(kt * BK);
+        store_tiles(kbeg + kt * BK);
         __syncthreads();
-        if (kt + 1 < ktiles) load_tiles((kt + 1) * BK);
+        if (kt + 1 < ktiles) load_tiles(kbeg + (kt + 1) * BK);
 
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 16) {

@@ -93,13 +93,30 @@ __global__ __launch_bounds__(256) void sp_gemv(const LayerArgs L, const float *_
         float wf[R][EPC];
 #pragma unroll
         for (int r = 0; r < R; ++r) unpack16<FMT>(wv[r], wf[r]);
+        // BF16 weights, three or four samples: left to itself the compiler waits for each sample's activations
+        // before it asks for the next one's (8192 x 8192: 65 us against 45 us for FP16 weights); all of a chunk's
+        // activation loads first, then the arithmetic
+        constexpr bool HOIST = FMT == BF16 && BT == 4;
+        float4 xs[HOIST ? BT : 1][HOIST ? EPC / 4 : 1];
+        if constexpr (HOIST) {
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                const int bb = b < nb ? b : nb - 1;
+                const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)c * EPC);
+#pragma unroll
+                for (int e = 0; e < EPC / 4; ++e) xs[b][e] = xp[e];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const int bb = b < nb ? b : nb - 1;
             const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)c * EPC);
 #pragma unroll
             for (int e = 0; e < EPC / 4; ++e) {
-                float4 xv = xp[e];
+                float4 xv;
+                if constexpr (HOIST) xv = xs[b][e];
+                else xv = xp[e];
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     acc[r][b] = fmaf(wf[r][4 * e + 0], xv.x, acc[r][b]);

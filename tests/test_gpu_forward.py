@@ -496,6 +496,30 @@ def test_split_mode_of_an_fp32_net_follows_new_weights(S, O):
     d.destroy()
 
 
+@pytest.mark.parametrize("fmt", ["f16", "bf16", "i8", "i4", "i2"])
+@pytest.mark.parametrize("n", [5, 64, 300])
+def test_rows_that_are_not_whole_16_byte_units_split_k_at_few_samples(S, O, fmt, n):
+    """Widths like 777 or 1030 keep every 16-bit and integer layer on the single-stage kernel with element-wise loads;
+    with few samples that is a handful of workgroups, so K is split over the grid (whole K tiles, partial sums added
+    in split order by a second launch).  Same tolerance as every matrix-core path, identical from call to call, with
+    plain and with split activations."""
+    topo, acts = [777, 1030, 515, 33], ["relu", "tanh", "none"]
+    src = make_oracle_net(O, topo, acts, seed=77, bias_std=0.1)
+    _, ref, net = quantized_pair(O, S, src, fmt)
+    X = np.random.default_rng(n).standard_normal((n, topo[0])).astype(F32)
+    want = ref.forward_batch_f64(X)
+    got = S.forward_batch(net, X)
+    again = S.forward_batch(net, X)
+    h = S.lib().spingalett_hip_handle(net)
+    assert S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() == "sp_gemm16"
+    assert S.lib().spingalett_set_net_activations(net, S.NET_ACTIVATIONS_SPLIT) == 0
+    fine = S.forward_batch(net, X)
+    S.free_network(net)
+    assert rel_max_abs(got, want) <= TOL_MFMA
+    assert np.array_equal(got, again)
+    assert rel_max_abs(fine, want) <= 2e-5
+
+
 def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
     """From five samples on the FP32 matrix-core kernel is the faster one for FP32 weights, as the 16-bit one is for
     the other formats (configuration 1 at 64 samples: 31 us against 245 us in eight passes of the vector kernel), and
