@@ -1056,6 +1056,11 @@ ThinPlan plan_thin(int fmt, uint32_t M, uint32_t N, uint32_t K)
     ThinPlan p{};
     if (N <= 64 && K % 8u == 0 && M >= 1) {
         p.use = true; p.mode_b = true; p.R = M; p.NC = N;
+    } else if (M >= 16u && (uint64_t)N * K <= (128u << 10)) {
+        // a layer of a few hundred rows and columns gives this kernel two or three workgroups, each fetching the whole
+        // thin operand before it starts: the single-stage tile kernel is quicker from 16 samples on (eight 256 x 256
+        // layers at 64 samples: 51 against 73-79 us in every format)
+        return p;
     } else if (M <= thin_max_samples(fmt, N, K) && rows_aligned(fmt, K) && K % 8u == 0) {
         p.use = true; p.mode_b = false; p.R = N; p.NC = M;
     } else {
@@ -1303,7 +1308,8 @@ void launch_gemm16(int fmt, const LayerArgs &L, const uint16_t *A, void *C, uint
     }
 }
 
-// K splits of the FP32 GEMM: enough workgroups for four per compute unit, at least two K tiles each
+// K splits of the FP32 GEMM: enough workgroups for four per compute unit, at least two K tiles each (also for tiny
+// layers: eight 256 x 256 layers at 5 .. 256 samples 58-62 us with the split and its second launch, 78-90 us without)
 uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 {
     const uint32_t tiles = ((M + 63) / 64) * ((N + 63) / 64), ktiles = (K + 31) / 32;
