@@ -1327,13 +1327,24 @@ uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, float *ws, uint64_t ws_floats, float *soft_out)
 {
     Gemm32Args g{L, A, C, nullptr, M, 0};
+    const bool vec = L.K % 4u == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(L.w) & 15u) == 0;
+    // weights beyond the L2s (4 MB per XCD) and enough 128 x 128 tiles for two per compute unit: the larger tile
+    if (vec && M >= 512u && (uint64_t)L.N * L.K * sizeof(float) > (4ull << 20) &&
+        (uint64_t)((M + 127u) / 128u) * ((L.N + 127u) / 128u) >= 512u) {
+        tl_route.name = "sp_gemm32_f32_big";
+        if (tl_route.dry) return false;
+        constexpr size_t lds = 2 * 2 * 128 * 36 * sizeof(float);
+        static bool once = ((void)hipFuncSetAttribute((const void *)sp_gemm32_f32_big, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+        (void)once;
+        sp_gemm32_f32_big<<<((M + 127u) / 128u) * ((L.N + 127u) / 128u), 256, lds, g_stream>>>(g);
+        return false;
+    }
     uint32_t splits = gemm32_splits(M, L.N, L.K, &g.kper);
     if (splits > 1 && (uint64_t)splits * M * L.N > ws_floats) { splits = 1; g.kper = (L.K + 31u) / 32u * 32u; }
     if (splits > 1) g.ws = ws;
     tl_route.name = "sp_gemm32_f32";
     if (tl_route.dry) return false;
     const dim3 grid(((M + 63) / 64) * ((L.N + 63) / 64), splits);
-    const bool vec = L.K % 4u == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && (reinterpret_cast<uintptr_t>(L.w) & 15u) == 0;
     if (vec) sp_gemm32_f32<true><<<grid, 256, 0, g_stream>>>(g);
     else sp_gemm32_f32<false><<<grid, 256, 0, g_stream>>>(g);
     if (splits > 1 && soft_out && L.N <= 64u) {

@@ -107,6 +107,108 @@ __global__ __launch_bounds__(256) void sp_gemm32_f32(const Gemm32Args g)
     }
 }
 
+// The same product for layers whose weights exceed the L2s, at 512 samples and more: 128 x 128 x 32 tile (each wave
+// 64 x 64 = 2 x 2 accumulators), two LDS stages and one barrier per K tile, rows of 36 floats in LDS.  MFMA step
+// (j, t), t = 0 .. 3, of a K tile multiplies k = 8 j + 4 h + t on the lanes of half h for both operands alike (a sum
+// over k in any order), so that a lane reads the four k of four steps with one 16-byte LDS load.  Half the bytes per
+// flop of the 64 x 64 tile, through LDS and through the fabric (8192 x 4096 x 4096: 9.2 GB fetched per launch with
+// 64 x 64 tiles).  Rows are 16-byte aligned (K % 4 == 0); no K split.
+__global__ __launch_bounds__(256) void sp_gemm32_f32_big(const Gemm32Args g)
+{
+    constexpr int BM = 128, BN = 128, BK = 32, LD = 36, SIZE = BM * LD;
+    extern __shared__ __attribute__((aligned(16))) float smem32[];
+    float *As = smem32, *Ws = smem32 + 2 * SIZE;
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1, q = lane & 31, h = lane >> 5;
+    const uint32_t tiles_n = (N + BN - 1) / BN;
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per = gridDim.x / 8u;          // each XCD a contiguous run of tiles
+        if (bid < per * 8u) bid = (bid & 7u) * per + (bid >> 3);
+    }
+    const uint32_t m0 = (bid / tiles_n) * BM, n0 = (bid % tiles_n) * BN;
+    const float *Wf = reinterpret_cast<const float *>(g.L.w);
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // piece p of a tile: row p / 8, k (p % 8) * 4; four pieces of A and of W per thread
+    float4 ra[4], rw[4];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = t + 256 * i;
+            const uint32_t row = (uint32_t)(p >> 3), k = k0 + (uint32_t)(p & 7) * 4u;
+            const uint32_t m = m0 + row, n = n0 + row;
+            const bool kin = k < K;
+            const float4 va = *reinterpret_cast<const float4 *>(g.A + (size_t)(m < M ? m : M - 1) * K + (kin ? k : 0u));
+            const float4 vw = *reinterpret_cast<const float4 *>(Wf + (size_t)(n < N ? n : N - 1) * K + (kin ? k : 0u));
+            ra[i] = (kin && m < M) ? va : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            rw[i] = (kin && n < N) ? vw : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    };
+    auto stash = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = t + 256 * i, o = (p >> 3) * LD + (p & 7) * 4;
+            *reinterpret_cast<float4 *>(As + stage * SIZE + o) = ra[i];
+            *reinterpret_cast<float4 *>(Ws + stage * SIZE + o) = rw[i];
+        }
+    };
+    auto compute = [&](int stage) {
+        const float *as = As + stage * SIZE + (wm * 64 + q) * LD + 4 * h, *ws = Ws + stage * SIZE + (wn * 64 + q) * LD + 4 * h;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float a[2][4], b[2][4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float4 va = *reinterpret_cast<const float4 *>(as + i * 32 * LD + 8 * j);
+                const float4 vb = *reinterpret_cast<const float4 *>(ws + i * 32 * LD + 8 * j);
+                a[i][0] = va.x; a[i][1] = va.y; a[i][2] = va.z; a[i][3] = va.w;
+                b[i][0] = vb.x; b[i][1] = vb.y; b[i][2] = vb.z; b[i][3] = vb.w;
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int jn = 0; jn < 2; ++jn) acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][tt], b[jn][tt], acc[i][jn], 0, 0, 0);
+        }
+    };
+
+    const uint32_t nk = (K + BK - 1) / BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        const bool more = kt + 1 < nk;
+        if (more) fetch((kt + 1) * BK);
+        compute((int)(kt & 1u));
+        if (more) stash((int)((kt + 1) & 1u));     // the other stage: every wave left it before the last barrier
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int jn = 0; jn < 2; ++jn) {
+        const uint32_t col = n0 + wn * 64 + jn * 32 + q;
+        if (col >= N) continue;
+        const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col) * g.L.bscale;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (row < M) g.C[(size_t)row * N + col] = apply_act(acc[i][jn][r] + bias, g.L.act);
+            }
+    }
+}
+
 // adds the K splits of sp_gemm32_f32 (in split order) and applies bias and activation
 __global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint32_t splits)
 {

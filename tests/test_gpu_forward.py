@@ -463,7 +463,7 @@ def test_split_mode_of_an_fp32_net_runs_on_the_16_bit_matrix_cores(S, O, topo, a
     assert rel_max_abs(again, want[:m]) <= 2e-5
     assert rel_max_abs(few, want[:64]) <= TOL_VEC
     assert [k.startswith(("sp_gemm16", "sp_skinny16")) for k in names] == [bool(x) for x in on16], names
-    assert all(k == "sp_gemm32_f32" for k, x in zip(names, on16) if not x), names
+    assert all(k.startswith("sp_gemm32_f32") for k, x in zip(names, on16) if not x), names
     if not any(on16):
         assert np.array_equal(got, plain)
 
@@ -518,6 +518,21 @@ def test_rows_that_are_not_whole_16_byte_units_split_k_at_few_samples(S, O, fmt,
     assert rel_max_abs(got, want) <= TOL_MFMA
     assert np.array_equal(got, again)
     assert rel_max_abs(fine, want) <= 2e-5
+
+
+def test_large_fp32_layers_take_the_128_by_128_tile(S, O):
+    """FP32 weights beyond the L2s at 512 samples and more: the two-stage 128 x 128 kernel (ragged M, N and a K that is
+    not a whole number of tiles), the layer behind it the 64 x 64 one; FP32 bar against the float64 forward."""
+    topo, acts, n = [1000, 1100, 300], ["tanh", "none"], 8195
+    src = make_oracle_net(O, topo, acts, seed=12, bias_std=0.1)
+    _, ref, net = quantized_pair(O, S, src, "f32")
+    h = S.lib().spingalett_hip_handle(net)
+    assert [S.lib().sphip_layer_kernel_name(h, l, n, 0).decode() for l in (1, 2)] == ["sp_gemm32_f32_big", "sp_gemm32_f32"]
+    assert S.lib().sphip_layer_kernel_name(h, 1, 500, 0).decode() == "sp_gemm32_f32"
+    X = np.random.default_rng(8).standard_normal((n, topo[0])).astype(F32)
+    got = S.forward_batch(net, X)
+    S.free_network(net)
+    assert rel_max_abs(got, ref.forward_batch_f64(X)) <= TOL_VEC
 
 
 def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
