@@ -802,12 +802,35 @@ template <int FMT>
 void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
 {
     const bool aligned = rows_aligned(FMT, L.K) && (L.K % 4u == 0);
-    tl_route.name = aligned ? "sp_gemv" : "sp_gemv_generic";
+    // integer rows of whole words: a word per lane when 16-byte chunks would leave most of a wave idle (rows of at
+    // most 16 chunks) or do not apply (rows that are not whole 16-byte units)
+    bool words = false;
+    uint32_t lpr = 64;
+    if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
+        const uint64_t row_bits = (uint64_t)L.K * fmt_bits(FMT);
+        // ... and for layers of at most 64 outputs, whose rows the 16-byte kernel would give to 32 waves or fewer:
+        // there a row of 256 words and more spans a whole workgroup (8192 -> 10 INT4 at four samples: 20 -> 11 us)
+        words = row_bits % 32u == 0 && (!aligned || row_bits <= 16u * 128u || L.N <= 64u) && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+        const uint32_t wpr = (uint32_t)(row_bits / 32u);
+        while (lpr > 1u && lpr / 2u >= wpr) lpr /= 2u;
+        if (L.N <= 64u && wpr >= 256u) lpr = 256u;
+    }
+    tl_route.name = words ? "sp_gemv_words" : aligned ? "sp_gemv" : "sp_gemv_generic";
     if (tl_route.dry) return;
     for (uint32_t b0 = 0; b0 < n; b0 += 8) {
         const int nb = (int)(n - b0 < 8 ? n - b0 : 8);
         const float *xb = x + (size_t)b0 * L.K;
         float *yb = y + (size_t)b0 * L.N;
+        if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
+            if (words) {
+                const uint32_t rows_per_wg = 256u / lpr, grid = (L.N + rows_per_wg - 1) / rows_per_wg;
+                if (nb == 1) sp_gemv_words<FMT, 1><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb, lpr);
+                else if (nb == 2) sp_gemv_words<FMT, 2><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb, lpr);
+                else if (nb <= 4) sp_gemv_words<FMT, 4><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb, lpr);
+                else sp_gemv_words<FMT, 8><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb, lpr);
+                continue;
+            }
+        }
         if (aligned) {
             constexpr int R = 2;
             const uint32_t waves = (L.N + R - 1) / R, grid = (waves + 3) / 4;
@@ -847,6 +870,9 @@ bool launch_gemv_i8(const Workspace &wk, const LayerArgs &L, const float *x, flo
     // 2.7 against 5.4 us at one sample and 4.4 against 7.3 us at four, 2048 x 2048 4.5 against 6.4 us at one; equal
     // from about 4 M code-sample products (INT2, whose decode costs more vector instructions: half that).
     if ((uint64_t)L.N * L.K * n <= (FMT == I2 ? (2ull << 20) : (4ull << 20))) return false;
+    // layers of at most 64 outputs are four row groups at most: the vector kernel with a workgroup per row is quicker
+    // (16384 -> 64 INT4 at four samples: 38 us here)
+    if (L.N <= 64u && n <= 4u) return false;
     if (reinterpret_cast<uintptr_t>(x) & 15u) return false;   // the quantiser reads float4
     const int need = (int)(n + 3) / 4;
     const int MT = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : need <= 12 ? 12 : 16;

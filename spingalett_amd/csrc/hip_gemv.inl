@@ -146,6 +146,75 @@ __global__ __launch_bounds__(256) void sp_gemv(const LayerArgs L, const float *_
     }
 }
 
+// Integer rows of whole 32-bit words, a word per lane: `lpr` lanes (a power of two) share a row, 64 / lpr rows per
+// wave.  For rows of a few hundred bytes, of which sp_gemv's 16-byte chunks occupy a handful of lanes (a 256-code INT2
+// row is four chunks), and for rows that are whole words but not whole 16-byte units (784 INT4 codes), which would
+// otherwise be fetched an element per lane.  K codes = K bits / 32 words; the activations of a word's codes are
+// 16-byte aligned (4, 8 or 16 floats).
+template <int FMT, int BT>
+__global__ __launch_bounds__(256) void sp_gemv_words(const LayerArgs L, const float *__restrict__ x, float *__restrict__ y, int nb,
+                                                     uint32_t lpr)
+{
+    constexpr int bits = fmt_bits(FMT), CW = 32 / bits;      // codes per word
+    const int lane = threadIdx.x & 63;
+    // lpr <= 64: 64 / lpr rows per wave; lpr = 128 or 256: a row spans two or four waves, whose sums meet in LDS
+    const uint32_t sub = threadIdx.x & (lpr - 1u);
+    const uint32_t row = lpr <= 64u ? (blockIdx.x * 4u + (threadIdx.x >> 6)) * (64u / lpr) + (uint32_t)lane / lpr
+                                    : blockIdx.x * (256u / lpr) + threadIdx.x / lpr;
+    const uint32_t wpr = L.K / CW;                            // words per row
+    const uint32_t rowc = row < L.N ? row : L.N - 1;
+    const uint32_t *wp = reinterpret_cast<const uint32_t *>(L.w) + (size_t)rowc * wpr;
+    float acc[BT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b) acc[b] = 0.0f;
+    for (uint32_t w = sub; w < wpr; w += lpr) {
+        const uint32_t word = wp[w];
+        float q[CW];
+#pragma unroll
+        for (int j = 0; j < CW; ++j) q[j] = (float)((int)(word << (32 - bits - bits * j)) >> (32 - bits));
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const int bb = b < nb ? b : nb - 1;
+            const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)w * CW);
+#pragma unroll
+            for (int e = 0; e < CW / 4; ++e) {
+                const float4 xv = xp[e];
+                acc[b] = fmaf(q[4 * e + 0], xv.x, acc[b]);
+                acc[b] = fmaf(q[4 * e + 1], xv.y, acc[b]);
+                acc[b] = fmaf(q[4 * e + 2], xv.z, acc[b]);
+                acc[b] = fmaf(q[4 * e + 3], xv.w, acc[b]);
+            }
+        }
+    }
+    for (uint32_t off = (lpr < 64u ? lpr : 64u) >> 1; off; off >>= 1) {
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[b] += __shfl_xor(acc[b], (int)off, kWave);
+    }
+    if (lpr > 64u) {                                          // (uniform over the workgroup)
+        __shared__ float part[4][BT];
+        const uint32_t wave = threadIdx.x >> 6, wpr_waves = lpr / 64u;
+        if (lane == 0) {
+#pragma unroll
+            for (int b = 0; b < BT; ++b) part[wave][b] = acc[b];
+        }
+        __syncthreads();
+        if (sub == 0) {
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float sum = part[wave][b];
+                for (uint32_t v = 1; v < wpr_waves; ++v) sum += part[wave + v][b];
+                acc[b] = sum;
+            }
+        }
+    }
+    if (sub == 0 && row < L.N) {
+        const float bias = elem_value_rt(L.bias_fmt, L.bias, row) * L.bscale;
+#pragma unroll
+        for (int b = 0; b < BT; ++b)
+            if (b < nb) y[(size_t)b * L.N + row] = apply_act(fmaf(acc[b], L.wscale, bias), L.act);
+    }
+}
+
 // Generic path: any K, rows may start inside a byte.  One wave per row, one
 // element per lane and step.
 template <int FMT, int BT>

@@ -746,7 +746,8 @@ def test_integer_matrix_core_gemv_forced_up_to_64_samples(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + K)
     # INT2 planes of more than 51 samples exceed the LDS of one fetch group: the vector kernel takes those
     fits = fmt != "i2" or n <= 51
-    assert _kernel_of(S, net, n, S.SPHIP_FORCE_GEMV) == ("sp_gemv_i8mfma" if fits else "sp_gemv")
+    vector = "sp_gemv_words" if K * {"i8": 8, "i2": 2}[fmt] <= 2048 else "sp_gemv"      # rows of at most 16 chunks: a word per lane
+    assert _kernel_of(S, net, n, S.SPHIP_FORCE_GEMV) == ("sp_gemv_i8mfma" if fits else vector)
     X = np.random.default_rng(n).standard_normal((n, K)).astype(F32)
     pre = X.astype(np.float64) @ W.T + b
     want = np.where(pre > 0, pre, 0.01 * pre)
@@ -760,8 +761,15 @@ def test_integer_matrix_core_gemv_forced_up_to_64_samples(S, fmt, N, K, n):
     ("i8", 2048, 2048, 1, "sp_gemv"), ("i8", 2064, 2048, 1, "sp_gemv_i8mfma"),
     ("i4", 1024, 1024, 4, "sp_gemv"), ("i4", 1040, 1024, 4, "sp_gemv_i8mfma"),
     ("i2", 1024, 2048, 1, "sp_gemv"), ("i2", 1040, 2048, 1, "sp_gemv_i8mfma"),
-    ("i2", 1024, 1024, 2, "sp_gemv"), ("i2", 1024, 1024, 3, "sp_gemv_i8mfma"),
-    ("i4", 4096, 2056, 2, "sp_gemv_generic"),          # rows that are not whole 16-byte units
+    ("i2", 1024, 1024, 2, "sp_gemv_words"), ("i2", 1024, 1024, 3, "sp_gemv_i8mfma"),
+    ("i2", 301, 250, 2, "sp_gemv_generic"),            # rows that are not whole 32-bit words
+    # rows of whole words: a word per lane when they are not whole 16-byte units, or at most 16 of them
+    ("i4", 4096, 2056, 2, "sp_gemv_words"), ("i2", 256, 256, 1, "sp_gemv_words"),
+    ("i4", 300, 264, 3, "sp_gemv_words"), ("i8", 100, 36, 4, "sp_gemv_words"), ("i2", 70, 16, 2, "sp_gemv_words"),
+    ("i4", 512, 784, 1, "sp_gemv_words"), ("i8", 33, 256, 4, "sp_gemv_words"),
+    # at most 64 outputs: a workgroup per row once a row has 256 words, whatever the layer's size
+    ("i4", 10, 8192, 4, "sp_gemv_words"), ("i4", 64, 16384, 3, "sp_gemv_words"), ("i2", 10, 8192, 2, "sp_gemv_words"),
+    ("i8", 7, 4100, 4, "sp_gemv_words"), ("i8", 64, 1024, 1, "sp_gemv_words"), ("i2", 65, 16384, 4, "sp_gemv_i8mfma"),
 ])
 def test_small_integer_layers_keep_the_vector_kernel(S, fmt, N, K, n, kernel):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=3 * N + K + n)
@@ -985,7 +993,7 @@ def test_integer_gemv_with_a_very_long_row_falls_back_to_the_vector_kernel(S):
     """A K so long that the self-quantising integer GEMV's two digit-plane buffers plus its scale records exceed the
     LDS of a compute unit (2 M columns at four samples: 64 KB of scale records next to two 48 KB plane buffers): the layer must route to the vector kernel, not fail at
     launch; and it must still compute the product."""
-    K, N, n = 1 << 21, 16, 4
+    K, N, n = 1 << 21, 80, 4                            # (more than 64 outputs: thinner layers never take that kernel)
     rng = np.random.default_rng(5)
     net = S.DeviceNet([K, N], [S.ACT_NONE], S.PRECISION_INT8)
     codes = rng.integers(-127, 128, size=N * K, dtype=np.int8)
