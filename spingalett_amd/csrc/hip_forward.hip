@@ -814,6 +814,10 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
         const uint32_t wpr = (uint32_t)(row_bits / 32u);
         while (lpr > 1u && lpr / 2u >= wpr) lpr /= 2u;
         if (L.N <= 64u && wpr >= 256u) lpr = 256u;
+    } else {
+        // FP32 and 16-bit weights: only the thin layers with long rows (a workgroup per row instead of a wave per two)
+        const uint64_t row_bits = (uint64_t)L.K * fmt_bits(FMT);
+        if (L.N <= 64u && row_bits % 32u == 0 && row_bits / 32u >= 256u) { words = true; lpr = 256u; }
     }
     tl_route.name = words ? "sp_gemv_words" : aligned ? "sp_gemv" : "sp_gemv_generic";
     if (tl_route.dry) return;
@@ -821,7 +825,7 @@ void launch_gemv_fmt(const LayerArgs &L, const float *x, float *y, uint32_t n)
         const int nb = (int)(n - b0 < 8 ? n - b0 : 8);
         const float *xb = x + (size_t)b0 * L.K;
         float *yb = y + (size_t)b0 * L.N;
-        if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
+        {
             if (words) {
                 const uint32_t rows_per_wg = 256u / lpr, grid = (L.N + rows_per_wg - 1) / rows_per_wg;
                 if (nb == 1) sp_gemv_words<FMT, 1><<<grid, 256, 0, g_stream>>>(L, xb, yb, nb, lpr);

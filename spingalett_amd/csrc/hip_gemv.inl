@@ -146,11 +146,11 @@ __global__ __launch_bounds__(256) void sp_gemv(const LayerArgs L, const float *_
     }
 }
 
-// Integer rows of whole 32-bit words, a word per lane: `lpr` lanes (a power of two) share a row, 64 / lpr rows per
-// wave.  For rows of a few hundred bytes, of which sp_gemv's 16-byte chunks occupy a handful of lanes (a 256-code INT2
+// Rows of whole 32-bit words, a word per lane: `lpr` lanes (a power of two) share a row, 64 / lpr rows per wave.  For rows of a few hundred bytes, of which sp_gemv's 16-byte chunks occupy a handful of lanes (a 256-code INT2
 // row is four chunks), and for rows that are whole words but not whole 16-byte units (784 INT4 codes), which would
-// otherwise be fetched an element per lane.  K codes = K bits / 32 words; the activations of a word's codes are
-// 16-byte aligned (4, 8 or 16 floats).
+// otherwise be fetched an element per lane.  K codes = K bits / 32 words; the activations of an integer word's codes
+// are 16-byte aligned (4, 8 or 16 floats).  FP32 and 16-bit rows (one or two values per word) come here for thin
+// layers only, a workgroup per row.
 template <int FMT, int BT>
 __global__ __launch_bounds__(256) void sp_gemv_words(const LayerArgs L, const float *__restrict__ x, float *__restrict__ y, int nb,
                                                      uint32_t lpr)
@@ -170,19 +170,39 @@ __global__ __launch_bounds__(256) void sp_gemv_words(const LayerArgs L, const fl
     for (uint32_t w = sub; w < wpr; w += lpr) {
         const uint32_t word = wp[w];
         float q[CW];
+        if constexpr (FMT == F32) {
+            q[0] = __uint_as_float(word);
+        } else if constexpr (FMT == F16) {
+            _Float16 lo, hi;
+            const uint16_t a = (uint16_t)(word & 0xFFFFu), b = (uint16_t)(word >> 16);
+            __builtin_memcpy(&lo, &a, 2);
+            __builtin_memcpy(&hi, &b, 2);
+            q[0] = (float)lo;
+            q[1] = (float)hi;
+        } else if constexpr (FMT == BF16) {
+            q[0] = __uint_as_float(word << 16);
+            q[1] = __uint_as_float(word & 0xFFFF0000u);
+        } else {
 #pragma unroll
-        for (int j = 0; j < CW; ++j) q[j] = (float)((int)(word << (32 - bits - bits * j)) >> (32 - bits));
+            for (int j = 0; j < CW; ++j) q[j] = (float)((int)(word << (32 - bits - bits * j)) >> (32 - bits));
+        }
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const int bb = b < nb ? b : nb - 1;
-            const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)bb * L.K + (size_t)w * CW);
+            const float *xw = x + (size_t)bb * L.K + (size_t)w * CW;
+            if constexpr (CW >= 4) {
+                const float4 *xp = reinterpret_cast<const float4 *>(xw);
 #pragma unroll
-            for (int e = 0; e < CW / 4; ++e) {
-                const float4 xv = xp[e];
-                acc[b] = fmaf(q[4 * e + 0], xv.x, acc[b]);
-                acc[b] = fmaf(q[4 * e + 1], xv.y, acc[b]);
-                acc[b] = fmaf(q[4 * e + 2], xv.z, acc[b]);
-                acc[b] = fmaf(q[4 * e + 3], xv.w, acc[b]);
+                for (int e = 0; e < CW / 4; ++e) {
+                    const float4 xv = xp[e];
+                    acc[b] = fmaf(q[4 * e + 0], xv.x, acc[b]);
+                    acc[b] = fmaf(q[4 * e + 1], xv.y, acc[b]);
+                    acc[b] = fmaf(q[4 * e + 2], xv.z, acc[b]);
+                    acc[b] = fmaf(q[4 * e + 3], xv.w, acc[b]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < CW; ++e) acc[b] = fmaf(q[e], xw[e], acc[b]);
             }
         }
     }

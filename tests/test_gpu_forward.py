@@ -545,6 +545,8 @@ def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
     h = S.lib().spingalett_hip_handle(net)
     assert [S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() for n in (1, 4, 5, 64, 65)] == \
         ["sp_gemv", "sp_gemv", "sp_gemm32_f32", "sp_gemm32_f32", "sp_gemm32_f32"]
+    # the 1000 -> 10 head: a workgroup per row at up to four samples
+    assert [S.lib().sphip_layer_kernel_name(h, 3, n, 0).decode() for n in (1, 4, 5)] == ["sp_gemv_words", "sp_gemv_words", "sp_gemm32_f32"]
     X = np.random.default_rng(3).random((64, topo[0]), dtype=F32)
     want = ref.forward_batch_f64(X)
     for n in (4, 5, 9, 33, 64):
@@ -770,6 +772,9 @@ def test_integer_matrix_core_gemv_forced_up_to_64_samples(S, fmt, N, K, n):
     # at most 64 outputs: a workgroup per row once a row has 256 words, whatever the layer's size
     ("i4", 10, 8192, 4, "sp_gemv_words"), ("i4", 64, 16384, 3, "sp_gemv_words"), ("i2", 10, 8192, 2, "sp_gemv_words"),
     ("i8", 7, 4100, 4, "sp_gemv_words"), ("i8", 64, 1024, 1, "sp_gemv_words"), ("i2", 65, 16384, 4, "sp_gemv_i8mfma"),
+    # ... 16-bit weights too (two values per word)
+    ("f16", 10, 8192, 4, "sp_gemv_words"), ("bf16", 64, 1000, 2, "sp_gemv_words"), ("bf16", 3, 514, 1, "sp_gemv_words"),
+    ("f16", 65, 8192, 4, "sp_gemv"), ("bf16", 10, 500, 3, "sp_gemv_generic"),
 ])
 def test_small_integer_layers_keep_the_vector_kernel(S, fmt, N, K, n, kernel):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=3 * N + K + n)
