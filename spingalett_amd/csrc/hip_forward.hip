@@ -1352,6 +1352,12 @@ uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
     return (ktiles + per - 1) / per;
 }
 
+// FP32 layers of at most 64 outputs are one row of tiles at most; with up to eight samples, one pass of the vector
+// kernel (a workgroup per row), that kernel is quicker than the matrix-core kernel and its reduction launch
+// (16384 -> 64 -> 10 at 5 / 8 samples: 24 / 25 against 43 us; 8192 -> 10: 13 against 23 us; at 16 samples, two passes,
+// 48 against 43 us.  Up to 64 K splits instead of 16 gave 32 us on the first and cost other thin layers 10 us.)
+bool f32_thin_vector(const LayerArgs &L, uint32_t n) { return L.N <= 64u && n <= 8u; }
+
 // soft_out: the layer is a softmax layer whose normalised outputs belong there; returns true if they were written
 // (a split-K layer of at most 64 outputs: the reduction does it), false if C holds the logits
 bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, float *ws, uint64_t ws_floats, float *soft_out)
@@ -1624,6 +1630,8 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
         if (run) {
             if (reg == R_GEMV) launch_gemv(net->prec, wk, L, (const float *)in, (float *)main_out, n, only_layer != 0 && net->aq_valid_layer == l && net->aq_valid_n == n);
             if (reg == R_GEMV) { net->aq_valid_layer = l; net->aq_valid_n = n; }
+            else if ((reg == R_GEMM32 || (reg == R_CAT3 && !cat3)) && f32_thin_vector(L, n))
+                launch_gemv(net->prec, wk, L, (const float *)in, (float *)main_out, n, false);
             else if (reg == R_GEMM32 || (reg == R_CAT3 && !cat3))
                 soft_done = launch_gemm32(L, (const float *)in, (float *)main_out, n, wk.split_ws, wk.split_cap,
                                           softmax && !only_layer ? (float *)dst : nullptr);
@@ -2289,11 +2297,13 @@ const char *sphip_layer_kernel_name(sphip_net *net, uint32_t layer, uint32_t n, 
         launch_gemv(net->prec, net->workspace(), L, aligned_ptr, nullptr, n, false);
         break;
     case R_GEMM32:
-        (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
+        if (f32_thin_vector(L, n)) launch_gemv(net->prec, net->workspace(), L, aligned_ptr, nullptr, n, false);
+        else (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
         break;
     case R_CAT3: {
         if (!cat3_layer(n, L.N, L.K)) {
-            (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
+            if (f32_thin_vector(L, n)) launch_gemv(net->prec, net->workspace(), L, aligned_ptr, nullptr, n, false);
+            else (void)launch_gemm32(L, aligned_ptr, nullptr, n, nullptr, ~0ull, nullptr);
             break;
         }
         LayerArgs L3 = L;

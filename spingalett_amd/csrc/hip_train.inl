@@ -540,7 +540,7 @@ int sphip_train_step(sphip_net *net, const float *x, const float *targets, uint3
         const bool softmax = net->act[l - 1] == A_SOFTMAX;
         float *main_out = softmax ? net->soft_tmp : ts->act[l];
         bool soft_done = false;
-        if (n <= kF32VectorMax) launch_gemv(net->prec, net->workspace(), L, in, main_out, n, false);
+        if (n <= kF32VectorMax || f32_thin_vector(L, n)) launch_gemv(net->prec, net->workspace(), L, in, main_out, n, false);
         else soft_done = launch_gemm32(L, in, main_out, n, net->split_ws, net->split_cap, softmax ? ts->act[l] : nullptr);
         if (softmax && !soft_done) sp_softmax_rows<<<(n + 3) / 4, 256, 0, g_stream>>>(net->soft_tmp, ts->act[l], 0, n, net->topo[l]);
         in = ts->act[l];

@@ -545,11 +545,12 @@ def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
     h = S.lib().spingalett_hip_handle(net)
     assert [S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() for n in (1, 4, 5, 64, 65)] == \
         ["sp_gemv", "sp_gemv", "sp_gemm32_f32", "sp_gemm32_f32", "sp_gemm32_f32"]
-    # the 1000 -> 10 head: a workgroup per row at up to four samples
-    assert [S.lib().sphip_layer_kernel_name(h, 3, n, 0).decode() for n in (1, 4, 5)] == ["sp_gemv_words", "sp_gemv_words", "sp_gemm32_f32"]
+    # the 1000 -> 10 head: a workgroup per row, up to eight samples (layers of at most 64 outputs)
+    assert [S.lib().sphip_layer_kernel_name(h, 3, n, 0).decode() for n in (1, 4, 5, 8, 9)] == \
+        ["sp_gemv_words"] * 4 + ["sp_gemm32_f32"]
     X = np.random.default_rng(3).random((64, topo[0]), dtype=F32)
     want = ref.forward_batch_f64(X)
-    for n in (4, 5, 9, 33, 64):
+    for n in (4, 5, 8, 9, 33, 64):
         assert rel_max_abs(S.forward_batch(net, X[:n]), want[:n]) <= TOL_VEC, n
     S.free_network(net)
 
