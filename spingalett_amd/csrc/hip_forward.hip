@@ -1250,8 +1250,13 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const uint32_t splits = gemm16_splits(FMT, M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * halves * M * L.N <= ctx.ws_floats;
     const bool halves_ok = halves == 1 || (uint64_t)halves * M * L.N <= ctx.ws_floats;     // (checked by the caller's reserve)
-    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok) && halves_ok) {
-        if (big_tiles >= 192u || !split_ok) g.kper = 0;
+    // (on a layer of up to 2 M weights a K split that still leaves fewer than 128 workgroups is no use of this kernel:
+    // 1024 x 1024 INT8 at 512 samples ran on 16 of them, eight K tiles each, 24 us a layer against 13 us on the
+    // single-stage kernel's 128 tiles; larger layers keep it, their workgroups walk a long K: 8192 x 8192 FP16 at 256
+    // samples 82 against 130 us)
+    const bool split_fills = split_ok && ((uint64_t)big_tiles * splits >= 128u || (uint64_t)L.N * L.K > (2u << 20));
+    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_fills) && halves_ok) {
+        if (big_tiles >= 192u) g.kper = 0;
         else g.ksplits = splits;
         if (g.kper || halves == 2) g.ws = ctx.ws;
         const dim3 grid(big_tiles, g.ksplits * halves);

@@ -652,7 +652,7 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     # Enough tiles for the chip (tails of 40, 8, 48 and 32 elements) ...
     ("bf16", 4096, 1000, 4096), ("f16", 4096, 1096, 3000), ("i8", 4096, 1008, 4096), ("i4", 4096, 1056, 4096),
     # ... K split over the grid, the partial tile in the last split ...
-    ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096), ("i4", 520, 1056, 300), ("i8", 1100, 2000, 700),
+    ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096), ("i4", 2080, 1056, 300), ("i8", 1100, 2000, 700),
     # ... a single row of 128 x 256 tiles, ragged in M and N, and a K of two tiles and a bit
     ("bf16", 8192, 1000, 100), ("f16", 5000, 1160, 77), ("bf16", 8200, 136, 8200),
     # output rows that are not whole 16-byte units: one element per lane and store, with and without a K split
@@ -820,7 +820,7 @@ def _same_nonfinite(got, want):
     ("i4", 512, 1024, 2, 0, "sp_gemv"), ("bf16", 600, 512, 4, 0, "sp_gemv"), ("i2", 301, 250, 3, 0, "sp_gemv_generic"),
     ("i4", 16384, 2048, 8, 0, "sp_skinny16_kw"), ("i8", 2100, 2064, 48, 0, "sp_skinny16"),
     ("f16", 1500, 1000, 77, 0, "sp_skinny16"), ("bf16", 10, 1000, 300, 0, "sp_skinny16_kw"),
-    ("bf16", 1024, 1024, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
+    ("bf16", 2048, 2048, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
     ("i8", 1000, 528, 700, 0, "sp_gemm16"), ("i4", 257, 100, 513, 0, "sp_gemm16"),
 ])
 def test_infinities_and_nans_travel_like_in_fp32(S, fmt, N, K, n, flags, kernel):
