@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void sp_train_out_delta(const float *__restric
 
 // Column sums of delta [n][width] (the sgemv against a vector of ones, Training.c:412-417) in two
 // passes: kColsumRows rows per workgroup into part[chunk][col], then the chunks in order, times scale.
-constexpr uint32_t kColsumRows = 1024;
+constexpr uint32_t kColsumRows = 256;
 __global__ __launch_bounds__(256) void sp_train_colsum_part(const float *__restrict__ d, float *__restrict__ part, uint32_t n,
                                                             uint32_t width)
 {
@@ -231,9 +231,15 @@ __global__ __launch_bounds__(256) void sp_train_colsum_fin(const float *__restri
 {
     const uint32_t col = blockIdx.x * 256u + threadIdx.x;
     if (col >= width) return;
-    float sum = 0.0f;
-    for (uint32_t ch = 0; ch < chunks; ++ch) sum += part[(size_t)ch * width + col];
-    out[col] = scale * sum;
+    // eight independent sums keep eight loads in flight (the chunks are added in a fixed order all the same)
+    float p[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t ch = 0;
+    for (; ch + 8u <= chunks; ch += 8u) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) p[u] += part[(size_t)(ch + u) * width + col];
+    }
+    for (; ch < chunks; ++ch) p[0] += part[(size_t)ch * width + col];
+    out[col] = scale * (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7])));
 }
 
 // Sum of squares of one array in FP64, one value per workgroup (first pass of clip_grad_norm, SIMD.c:496-520)
