@@ -46,6 +46,8 @@ CASES = [
     ("f32", [96, 160, 10], ["foo52", "softmax"], (64, 1), 0),
     ("i4", [256, 512, 384, 40], ["relu", "tanh", "softmax"], (300, 9), 128),       # split activations: partial sums of both matrices
     ("bf16", [512, 1024, 1000], ["leaky_relu", "softmax"], (2048, 70), 128),
+    ("i8", [777, 1030, 515, 33], ["relu", "tanh", "none"], (64, 5), 0),            # ragged rows: K split of the single-stage kernel
+    ("i2", [256, 256, 256, 64, 10], ["relu", "relu", "tanh", "softmax"], (3, 1), 0),   # word-per-lane vector kernel
 ]
 
 
