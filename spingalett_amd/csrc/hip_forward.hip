@@ -1363,6 +1363,13 @@ uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 // 48 against 43 us.  Up to 64 K splits instead of 16 gave 32 us on the first and cost other thin layers 10 us.)
 bool f32_thin_vector(const LayerArgs &L, uint32_t n) { return L.N <= 64u && n <= 8u; }
 
+// Unused dynamic LDS for the 64 x 64 FP32 forward kernel when the grid is several times what the chip holds: with
+// 32 KB per workgroup five of them share a compute unit instead of eight, and a product of thousands of tiles runs
+// 3-5 % faster (20000 x 1000 x 512: 221 -> 210 us standalone, 227 -> 220 us in the training step; 20000 x 512 x 784:
+// 179 -> 175 us; more padding, four per compute unit: the same).  The training products with their other operand
+// layouts lose by it (235 -> 240 us, and 48 -> 53 us where K is 10 and memory decides).  `own`: the kernel's static LDS.
+size_t gemm32_lds_pad(uint64_t workgroups, size_t own) { return workgroups >= 2048u && own < (32u << 10) ? (32u << 10) - own : 0; }
+
 // soft_out: the layer is a softmax layer whose normalised outputs belong there; returns true if they were written
 // (a split-K layer of at most 64 outputs: the reduction does it), false if C holds the logits
 bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, float *ws, uint64_t ws_floats, float *soft_out)
@@ -1386,8 +1393,9 @@ bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, flo
     tl_route.name = "sp_gemm32_f32";
     if (tl_route.dry) return false;
     const dim3 grid(((M + 63) / 64) * ((L.N + 63) / 64), splits);
-    if (vec) sp_gemm32_f32<true><<<grid, 256, 0, g_stream>>>(g);
-    else sp_gemm32_f32<false><<<grid, 256, 0, g_stream>>>(g);
+    const size_t pad = gemm32_lds_pad((uint64_t)grid.x * grid.y, 17u << 10);
+    if (vec) sp_gemm32_f32<true><<<grid, 256, pad, g_stream>>>(g);
+    else sp_gemm32_f32<false><<<grid, 256, pad, g_stream>>>(g);
     if (splits > 1 && soft_out && L.N <= 64u) {
         sp_gemm32_reduce_softmax<<<(M + 15u) / 16u, 256, 0, g_stream>>>(g, splits, soft_out);
         return true;
