@@ -220,6 +220,74 @@ __global__ __launch_bounds__(256) void sp_gemm32_f32_big(const Gemm32Args g)
     }
 }
 
+// Small FP32 layers in one launch: a workgroup owns a 32 x 32 tile of the output, its eight waves split K in whole
+// steps of eight, and their sums meet in LDS.  No operand staging: lane (r, h) loads four consecutive k of row r of both
+// operands (k = 8 s + 4 h .. + 3 of step s) straight into registers and feeds them to four MFMA steps (a sum over k in
+// any order).  For outputs of up to 512 tiles and K up to 1024, where sp_gemm32_f32 needs a K split over the grid and a
+// second launch to fill the chip (256 x 512 x 784: 8 us against 12 us for the two).  A softmax layer of at most 32
+// outputs is normalised here (Activation.c:5-21), soft_out != nullptr.  Rows are 16-byte aligned (K % 4 == 0).
+__global__ __launch_bounds__(512) void sp_gemm32_small(const Gemm32Args g, float *__restrict__ soft_out)
+{
+    constexpr int NW = 8, U = 4;
+    __shared__ float part[NW][32 * 33];
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, q = lane & 31, h = lane >> 5;
+    const uint32_t tiles_n = (N + 31u) / 32u;
+    const uint32_t m0 = (blockIdx.x / tiles_n) * 32u, n0 = (blockIdx.x % tiles_n) * 32u;
+    const uint32_t steps = (K + 7u) / 8u, per = (steps + NW - 1) / NW;
+    const uint32_t s0 = wave * per, s1 = s0 + per < steps ? s0 + per : steps;
+    const uint32_t am = m0 + q < M ? m0 + q : M - 1, wn = n0 + q < N ? n0 + q : N - 1;
+    const float *ap = g.A + (size_t)am * K + 4 * h;
+    const float *wp = reinterpret_cast<const float *>(g.L.w) + (size_t)wn * K + 4 * h;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    auto ld = [&](const float *p, uint32_t s) -> float4 {       // K % 4 == 0: a piece is inside the row or beyond it
+        return 8u * s + 4u * h < K ? *reinterpret_cast<const float4 *>(p + 8u * s) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    };
+    auto fma4 = [&](const float4 &a, const float4 &b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+    };
+    uint32_t s = s0;
+    for (; s + U <= s1; s += U) {
+        float4 a[U], b[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { a[u] = ld(ap, s + u); b[u] = ld(wp, s + u); }
+#pragma unroll
+        for (int u = 0; u < U; ++u) fma4(a[u], b[u]);
+    }
+    for (; s < s1; ++s) fma4(ld(ap, s), ld(wp, s));
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave][(8 * (r >> 2) + 4 * h + (r & 3)) * 33 + q] = acc[r];
+    __syncthreads();
+    // the waves' sums in wave order, bias, activation; 512 threads, two outputs each
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = t + 512 * i, row = e >> 5, col = e & 31;
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += part[w][row * 33 + col];
+        const uint32_t n = n0 + col < N ? n0 + col : N - 1;
+        v = apply_act(v + elem_value_rt(g.L.bias_fmt, g.L.bias, n) * g.L.bscale, g.L.act);
+        if (soft_out) part[0][row * 33 + col] = v;               // (every thread has read part[0][its own two slots] only)
+        else if (m0 + row < M && n0 + col < N) g.C[(size_t)(m0 + row) * N + n0 + col] = v;
+    }
+    if (!soft_out) return;                                        // (uniform)
+    __syncthreads();
+    if (t < 32 && m0 + t < M) {                                   // N <= 32: the tile holds whole rows of logits
+        const float *lr = &part[0][t * 33];
+        float mx = lr[0];
+        for (uint32_t c = 1; c < N; ++c) mx = fmaxf(mx, lr[c]);
+        float sum = 0.0f;
+        for (uint32_t c = 0; c < N; ++c) sum += expf(lr[c] - mx);
+        const float inv = sum > 0.0f ? 1.0f / sum : 1.0f;
+        for (uint32_t c = 0; c < N; ++c) soft_out[(size_t)(m0 + t) * N + c] = expf(lr[c] - mx) * inv;
+    }
+}
+
 // adds the K splits of sp_gemm32_f32 (in split order) and applies bias and activation
 __global__ __launch_bounds__(256) void sp_gemm32_reduce(const Gemm32Args g, uint32_t splits)
 {

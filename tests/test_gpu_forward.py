@@ -463,7 +463,7 @@ def test_split_mode_of_an_fp32_net_runs_on_the_16_bit_matrix_cores(S, O, topo, a
     assert rel_max_abs(again, want[:m]) <= 2e-5
     assert rel_max_abs(few, want[:64]) <= TOL_VEC
     assert [k.startswith(("sp_gemm16", "sp_skinny16")) for k in names] == [bool(x) for x in on16], names
-    assert all(k.startswith("sp_gemm32_f32") for k, x in zip(names, on16) if not x), names
+    assert all(k.startswith("sp_gemm32") for k, x in zip(names, on16) if not x), names
     if not any(on16):
         assert np.array_equal(got, plain)
 
@@ -543,14 +543,15 @@ def test_fp32_nets_leave_the_vector_kernel_beyond_four_samples(S, O):
     src = make_oracle_net(O, topo, acts, seed=5, bias_std=0.1)
     _, ref, net = quantized_pair(O, S, src, "f32")
     h = S.lib().spingalett_hip_handle(net)
-    assert [S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() for n in (1, 4, 5, 64, 65)] == \
-        ["sp_gemv", "sp_gemv", "sp_gemm32_f32", "sp_gemm32_f32", "sp_gemm32_f32"]
+    # (512 x 784 at these batch sizes: the one-launch kernel for small layers; at 4096 samples the tiled one)
+    assert [S.lib().sphip_layer_kernel_name(h, 1, n, 0).decode() for n in (1, 4, 5, 64, 65, 4096)] == \
+        ["sp_gemv", "sp_gemv", "sp_gemm32_small", "sp_gemm32_small", "sp_gemm32_small", "sp_gemm32_f32"]
     # the 1000 -> 10 head: a workgroup per row, up to eight samples (layers of at most 64 outputs)
     assert [S.lib().sphip_layer_kernel_name(h, 3, n, 0).decode() for n in (1, 4, 5, 8, 9)] == \
-        ["sp_gemv_words"] * 4 + ["sp_gemm32_f32"]
-    X = np.random.default_rng(3).random((64, topo[0]), dtype=F32)
+        ["sp_gemv_words"] * 4 + ["sp_gemm32_small"]
+    X = np.random.default_rng(3).random((4096, topo[0]), dtype=F32)
     want = ref.forward_batch_f64(X)
-    for n in (4, 5, 8, 9, 33, 64):
+    for n in (4, 5, 8, 9, 33, 64, 300, 4096):
         assert rel_max_abs(S.forward_batch(net, X[:n]), want[:n]) <= TOL_VEC, n
     S.free_network(net)
 
