@@ -1049,6 +1049,7 @@ struct ThinCtx {
     const uint16_t *w16;   // [N][K] 16-bit weights (raw 16-bit formats, or FP16 codes) when N <= 64, else nullptr
     float *ws;             // split-K workspace
     uint64_t ws_floats;
+    bool x_f32;            // A is still the caller's FP32 input (the layer is one gemm16_small_layer() accepts)
     void *soft_out;        // softmax layer: where the normalised outputs go if the layer's kernel can do it itself ...
     int soft_kind;         // ... as 0 FP32, 1 BF16, 2 FP16
     bool *soft_done;       // ... and whether it did
@@ -1214,11 +1215,35 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
     }
 }
 
+// Layers that run in one launch of sp_gemm16_small: more than 8 samples (fewer take one launch of sp_skinny16_kw), more
+// than 64 outputs (fewer stream the activations), at most 512 tiles of 32 x 32, K up to 2048 (its eight waves are all
+// the K split there is), and tiles x K up to 512 K: every tile reads 64 rows of K elements from L2.  Measured, whole
+// nets, against the streaming / tiled kernels with their K split over the grid, second launch and separate conversion
+// of the input: 784-512-1000-10 INT8 at 16 / 256 / 512 samples 16.5 / 18.9 / 22.3 against 24.8 / 29.8 / 28.0 us, eight
+// 256 x 256 layers at 64 / 1024 samples 31 / 35 against 51 / 49 us, three 1024 x 1024 layers at 256 samples 24 against
+// 38 us, at 512 samples (512 tiles x 1024) 40 against 41 us; beyond the bound it loses: two 2048 x 2048 layers at 256
+// samples (512 tiles x 2048) 46 against 35 us.
+bool gemm16_small_layer(uint32_t M, uint32_t N, uint32_t K, uint32_t halves)
+{
+    if (halves != 1u || K % 8u != 0 || K > 2048u || N <= 64u || M <= 8u) return false;
+    const uint64_t tiles = (uint64_t)((M + 31u) / 32u) * ((N + 31u) / 32u);
+    return tiles <= 512u && tiles * K <= (512u << 10);
+}
+
 template <int FMT, bool F16T>
 void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t M, int out_f32, const ThinCtx &ctx)
 {
-    const ThinPlan tp = plan_thin(FMT, M, L.N, L.K);
     const uint32_t halves = tl_route.halves;
+    if (gemm16_small_layer(M, L.N, L.K, halves) && (reinterpret_cast<uintptr_t>(A) & 15u) == 0) {
+        GemmArgs g{L, A, C, M, out_f32, nullptr, 0, 1, 1};
+        tl_route.name = "sp_gemm16_small";
+        if (tl_route.dry) return;
+        const uint32_t grid = ((M + 31u) / 32u) * ((L.N + 31u) / 32u);
+        if (ctx.x_f32) sp_gemm16_small<FMT, F16T, true><<<grid, 512, 0, g_stream>>>(g);
+        else sp_gemm16_small<FMT, F16T, false><<<grid, 512, 0, g_stream>>>(g);
+        return;
+    }
+    const ThinPlan tp = plan_thin(FMT, M, L.N, L.K);
     if (tp.use && (!tp.mode_b || ctx.w16) &&
         ((tp.splits == 1 && halves == 1) || (uint64_t)tp.splits * halves * tp.NC * tp.R <= ctx.ws_floats)) {
         SkinnyArgs a{};
@@ -1615,10 +1640,14 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
     const uint32_t last = net->layers - 1;
 
     const void *in = d_x;
+    const bool x_fused = reg == R_GEMM16 && gemm16_small_layer(n, net->topo[1], net->topo[0], tl_route.halves) &&
+                         (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0;
     if (split && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         sp_cvt16_split<<<(uint32_t)((cnt / 4 + 255) / 256 + 1), 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
         in = wk.buf[1];
+    } else if (x_fused) {
+        // (the first layer's kernel rounds the FP32 input itself)
     } else if (reg == R_GEMM16 && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         const uint32_t grid = (uint32_t)((cnt / 4 + 255) / 256 + 1);
@@ -1681,6 +1710,7 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
                 else ctx.w16 = wk.codes16[l - 1];
                 ctx.ws = wk.split_ws;
                 ctx.ws_floats = wk.split_cap;
+                ctx.x_f32 = x_fused && l == 1;
                 if (softmax && !only_layer) {
                     ctx.soft_out = dst;
                     ctx.soft_kind = !is_last ? (split ? 3 : f16t ? 2 : 1) : 0;

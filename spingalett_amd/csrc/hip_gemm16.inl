@@ -355,6 +355,123 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     else emit(std::false_type{});
 }
 
+// Small layers in one launch: a workgroup owns a 32 x 32 tile of the output, its eight waves split K in whole steps of
+// 32, and their sums meet in LDS.  No operand staging: in step s lane (r, h) loads the sixteen consecutive elements
+// k = 32 s + 16 h .. + 15 of row r of both operands straight into registers, as two pieces of eight (K % 8 == 0: a piece
+// is inside its row or beyond it), and feeds a piece of each operand to one MFMA (a sum over k in any order).  For
+// outputs of a few hundred tiles, where the streaming and the tiled kernels need a K split over the grid and a second
+// launch to fill the chip.  XF32: the activations are still the caller's FP32 input, rounded here as sp_cvt16 would
+// (g.A then points at floats).
+template <int FMT, bool F16T, bool XF32>
+__global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
+{
+    constexpr int NW = 8, U = 2;
+    constexpr int bits = fmt_bits(FMT);
+    constexpr int PB = bits;                           // bytes of a piece of eight weights
+    __shared__ float part[NW][32 * 33];
+    const uint32_t M = g.M, N = g.L.N, K = g.L.K;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, q = lane & 31, h = lane >> 5;
+    const uint32_t tiles_n = (N + 31u) / 32u;
+    const uint32_t m0 = (blockIdx.x / tiles_n) * 32u, n0 = (blockIdx.x % tiles_n) * 32u;
+    const uint32_t steps = (K + 31u) / 32u, per = (steps + NW - 1) / NW;
+    const uint32_t s0 = wave * per, s1 = s0 + per < steps ? s0 + per : steps;
+    const uint32_t am = m0 + q < M ? m0 + q : M - 1, wn = n0 + q < N ? n0 + q : N - 1;
+    const uint16_t *ap16 = g.A + (size_t)am * K + 16 * h;
+    const float *ap32 = reinterpret_cast<const float *>(g.A) + (size_t)am * K + 16 * h;
+    const uint8_t *wp = g.L.w + (size_t)wn * ((size_t)K * bits / 8u) + (size_t)(2 * h) * PB;
+
+    struct Frag { uint4 a[2], w[2]; };
+    auto ld = [&](uint32_t s) -> Frag {
+        Frag f;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const bool ok = 32u * s + 16u * h + 8u * p < K;
+            if constexpr (XF32) {
+                const float4 lo = ok ? *reinterpret_cast<const float4 *>(ap32 + 32u * s + 8 * p) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                const float4 hi = ok ? *reinterpret_cast<const float4 *>(ap32 + 32u * s + 8 * p + 4) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                f.a[p].x = (uint32_t)f32_to_t16<F16T>(lo.x) | ((uint32_t)f32_to_t16<F16T>(lo.y) << 16);
+                f.a[p].y = (uint32_t)f32_to_t16<F16T>(lo.z) | ((uint32_t)f32_to_t16<F16T>(lo.w) << 16);
+                f.a[p].z = (uint32_t)f32_to_t16<F16T>(hi.x) | ((uint32_t)f32_to_t16<F16T>(hi.y) << 16);
+                f.a[p].w = (uint32_t)f32_to_t16<F16T>(hi.z) | ((uint32_t)f32_to_t16<F16T>(hi.w) << 16);
+            } else {
+                f.a[p] = ok ? *reinterpret_cast<const uint4 *>(ap16 + 32u * s + 8 * p) : make_uint4(0, 0, 0, 0);
+            }
+            const uint8_t *src = wp + (size_t)s * (4 * PB) + p * PB;
+            if constexpr (FMT == F16 || FMT == BF16) {
+                f.w[p] = ok ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+            } else if constexpr (FMT == I8) {
+                const uint2 c = ok ? *reinterpret_cast<const uint2 *>(src) : make_uint2(0, 0);
+                f.w[p].x = c.x; f.w[p].y = c.y;
+            } else if constexpr (FMT == I4) {
+                f.w[p].x = ok ? *reinterpret_cast<const uint32_t *>(src) : 0u;
+            } else {
+                f.w[p].x = ok ? (uint32_t)*reinterpret_cast<const uint16_t *>(src) : 0u;
+            }
+        }
+        return f;
+    };
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    auto fma2 = [&](const Frag &f) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            uint4 wv = f.w[p];
+            if constexpr (FMT == I8) {
+                uint32_t o[4];
+                unpack_word16<I8, F16T>(f.w[p].x, o);
+                unpack_word16<I8, F16T>(f.w[p].y, o + 2);
+                wv = make_uint4(o[0], o[1], o[2], o[3]);
+            } else if constexpr (FMT == I4) {
+                uint32_t o[4];
+                unpack_word16<I4, F16T>(f.w[p].x, o);
+                wv = make_uint4(o[0], o[1], o[2], o[3]);
+            } else if constexpr (FMT == I2) {
+                uint32_t o[8];                          // (the upper eight codes of the word are not there: zeros)
+                unpack_word16<I2, F16T>(f.w[p].x, o);
+                wv = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+            if constexpr (F16T) {
+                f16x8 a, b;
+                __builtin_memcpy(&a, &f.a[p], 16);
+                __builtin_memcpy(&b, &wv, 16);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+            } else {
+                bf16x8 a, b;
+                __builtin_memcpy(&a, &f.a[p], 16);
+                __builtin_memcpy(&b, &wv, 16);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+            }
+        }
+    };
+    uint32_t s = s0;
+    for (; s + U <= s1; s += U) {
+        Frag f[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) f[u] = ld(s + u);
+#pragma unroll
+        for (int u = 0; u < U; ++u) fma2(f[u]);
+    }
+    for (; s < s1; ++s) fma2(ld(s));
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave][(8 * (r >> 2) + 4 * h + (r & 3)) * 33 + q] = acc[r];
+    __syncthreads();
+    // the waves' sums in wave order, scale, bias, activation; 512 threads, two outputs each
+    const float wscale = g.L.wscale;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = t + 512 * i, row = e >> 5, col = e & 31;
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += part[w][row * 33 + col];
+        if (m0 + row >= M || n0 + col >= N) continue;
+        v = apply_act(fmaf(v, wscale, elem_value_rt(g.L.bias_fmt, g.L.bias, n0 + col) * g.L.bscale), g.L.act);
+        const size_t o = (size_t)(m0 + row) * N + n0 + col;
+        if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
+        else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+    }
+}
+
 template <int OFF>
 __device__ __forceinline__ void ds_read128(u32x4 &dst, uint32_t addr);
 

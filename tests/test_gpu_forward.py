@@ -630,12 +630,13 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     # Too few 256 x 256 tiles and too few K tiles to split K over the grid: the single-stage tiled GEMM; by tile
     # count it runs 64 x 64, 64 x 128 or 128 x 128 tiles (ragged edges in both directions), rows that are not whole
     # 16-byte units take the element-wise loads and always 64 x 64
-    ("bf16", 512, 784, 600), ("i8", 1000, 528, 4096),
+    # (more than 512 tiles of 32 x 32, or more than 512 K of tiles x K: fewer go to the one-launch kernel below)
+    ("bf16", 512, 784, 1200), ("i8", 1000, 528, 4096),
     ("i2", 2048, 1056, 2048),
-    ("i8", 300, 1000, 700), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 512),
+    ("i8", 300, 1000, 1800), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 2400),
     # integer rows that are whole 32-bit words but not whole 16-byte units (784 INT4 codes = 392 bytes): word loads
-    ("i4", 512, 784, 1024), ("i2", 300, 784, 300), ("i8", 1000, 776, 600), ("i4", 520, 1000, 64), ("i2", 2048, 1008, 2048),
-    ("i4", 70, 24, 9), ("i8", 4096, 72, 4096),
+    ("i4", 512, 784, 2048), ("i2", 300, 784, 2000), ("i8", 1000, 776, 600), ("i4", 520, 1000, 1100), ("i2", 2048, 1008, 2048),
+    ("i4", 70, 24, 8), ("i8", 4096, 72, 4096),
 ])
 def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
@@ -645,6 +646,30 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     got = net.forward(X)
     assert _kernel_of(S, net, n) == "sp_gemm16"
     assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
+    net.destroy()
+
+
+@pytest.mark.parametrize("fmt,N,K,n", [
+    # up to 512 tiles of 32 x 32 and K up to 2048: ragged edges in both directions, K tails of 8, 16 and 24 elements
+    # (K = 1000, 784, 24, 72), a K shorter than the eight waves' shares, every weight format, 9 samples and up
+    ("bf16", 512, 784, 600), ("i8", 300, 1000, 700), ("i8", 200, 1000, 512), ("i4", 512, 784, 1024), ("i2", 300, 784, 300),
+    ("i4", 520, 1000, 64), ("i4", 70, 24, 9), ("f16", 1500, 1000, 77), ("i2", 1000, 320, 130), ("bf16", 4096, 2048, 40),
+    ("i8", 512, 784, 256), ("i8", 1000, 512, 256), ("f16", 65, 8, 9), ("i2", 97, 2048, 33), ("bf16", 16384, 32, 32),
+    ("i8", 256, 256, 2048), ("f16", 1024, 1024, 512), ("i4", 2048, 2048, 128), ("i2", 130, 72, 1000),
+])
+def test_small_layers_run_in_one_launch(S, fmt, N, K, n):
+    """Layers of a few hundred 32 x 32 output tiles run in one launch whose workgroups split K among their waves and
+    round the FP32 input themselves (no K split over the grid, no second launch, no separate conversion); checked
+    against FP64 on the decoded arrays."""
+    net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 5 * K + n)
+    X = np.random.default_rng(n + 2).standard_normal((n, K)).astype(F32)
+    pre = X.astype(np.float64) @ W.T + b
+    want = np.where(pre > 0, pre, 0.01 * pre)
+    got = net.forward(X)
+    assert _kernel_of(S, net, n) == "sp_gemm16_small"
+    assert rel_max_abs(got, want) <= (4e-3 if fmt == "bf16" else 1e-3)
+    if fmt == "bf16":                                # BF16 activations against the BF16 weights themselves
+        assert rel_max_abs(net.forward(X, S.SPHIP_BF16_ACTIVATIONS), want) <= 1e-2
     net.destroy()
 
 
@@ -820,7 +845,8 @@ def _same_nonfinite(got, want):
     ("i2", 8192, 8192, 4, 0, "sp_gemv_i8mfma"), ("i8", 1030, 1040, 17, 16, "sp_gemv_i8mfma"),
     ("i4", 512, 1024, 2, 0, "sp_gemv"), ("bf16", 600, 512, 4, 0, "sp_gemv"), ("i2", 301, 250, 3, 0, "sp_gemv_generic"),
     ("i4", 16384, 2048, 8, 0, "sp_skinny16_kw"), ("i8", 2100, 2064, 48, 0, "sp_skinny16"),
-    ("f16", 1500, 1000, 77, 0, "sp_skinny16"), ("bf16", 10, 1000, 300, 0, "sp_skinny16_kw"),
+    ("f16", 1500, 4096, 60, 0, "sp_skinny16"), ("bf16", 10, 1000, 300, 0, "sp_skinny16_kw"),
+    ("f16", 1500, 1000, 77, 0, "sp_gemm16_small"), ("i2", 600, 1000, 200, 0, "sp_gemm16_small"),
     ("bf16", 2048, 2048, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
     ("i8", 1000, 528, 700, 0, "sp_gemm16"), ("i4", 257, 100, 513, 0, "sp_gemm16"),
 ])
