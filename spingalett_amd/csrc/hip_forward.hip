@@ -1012,13 +1012,18 @@ uint32_t gemm16_tile_rows(int fmt, uint32_t M, uint32_t N)
     return ((M + 255u) / 256u) * cols < 192u && ((M + 127u) / 128u) * cols <= 256u ? 128u : 256u;
 }
 
-// K splits of the tile GEMM when its tiles would leave compute units idle: at least eight K tiles each
+// K splits of the tile GEMM when its tiles would leave compute units idle: from K = 4096 on (16-bit weights, which reach
+// LDS by DMA: 3072), at least eight K tiles each.  Below, the single-stage kernel's small tiles fill the chip in one launch and no partial sums travel (forward
+// of one layer, conversion of the input included, K split here against single stage: 4096 x 512 x 1024 FP16 24.8
+// against 13.3 us, 1024 x 4096 x 1024 32.6 against 26.1 us, 1024 x 2048 x 2048 31.1 against 26.0 us, INT8 34.4 against
+// 27.3 us; at K = 3072 FP16 128 x 4096 x 3072 21.7 against 26.9 us, 1024 x 2048 x 3072 even, INT8 40.5 against 37.6 us; from
+// K = 4096 the long walk pays: 512 x 2048 x 4096 30.4 against 37.1 us, 256 x 8192 x 8192 53 against 82 us)
 uint32_t gemm16_splits(int fmt, uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
 {
     const uint32_t bm = gemm16_tile_rows(fmt, M, N);
     const uint32_t tiles = ((M + bm - 1) / bm) * ((N + 255u) / 256u), ktiles = (K + 63u) / 64u;
     *kper = 0;
-    if (tiles >= 192u || ktiles < 16u) return 1;
+    if (tiles >= 192u || ktiles < (fmt_bits(fmt) == 16 ? 48u : 64u)) return 1;
     uint32_t splits = (256u + tiles - 1) / tiles;
     if (splits > 8u) splits = 8u;
     if (splits > ktiles / 8u) splits = ktiles / 8u;
@@ -1275,12 +1280,8 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     const uint32_t splits = gemm16_splits(FMT, M, L.N, L.K, &g.kper);
     const bool split_ok = splits > 1 && (uint64_t)splits * halves * M * L.N <= ctx.ws_floats;
     const bool halves_ok = halves == 1 || (uint64_t)halves * M * L.N <= ctx.ws_floats;     // (checked by the caller's reserve)
-    // (on a layer of up to 2 M weights a K split that still leaves fewer than 128 workgroups is no use of this kernel:
-    // 1024 x 1024 INT8 at 512 samples ran on 16 of them, eight K tiles each, 24 us a layer against 13 us on the
-    // single-stage kernel's 128 tiles; larger layers keep it, their workgroups walk a long K: 8192 x 8192 FP16 at 256
-    // samples 82 against 130 us)
-    const bool split_fills = split_ok && ((uint64_t)big_tiles * splits >= 128u || (uint64_t)L.N * L.K > (2u << 20));
-    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_fills) && halves_ok) {
+    // (too few tiles and no K split, gemm16_splits: the single-stage kernel below)
+    if (aligned && L.K >= 128u && M > 64 && L.N >= 256 && fits32 && (big_tiles >= 192u || split_ok) && halves_ok) {
         if (big_tiles >= 192u) g.kper = 0;
         else g.ksplits = splits;
         if (g.kper || halves == 2) g.ws = ctx.ws;
@@ -1331,9 +1332,24 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((L.N + bn - 1) / bn); };
     // (words: integer codes whose rows are whole 32-bit words, not whole 16-byte units, next to aligned activations)
     const int shape = !(aligned || words) ? 11 : tiles(128, 128) >= 512u ? 22 : tiles(64, 128) >= 512u ? 12 : 11;
+    // K of 1024 and more: K tiles of 128 instead of 64, half as many rounds of load, barrier, store, barrier (600 x 1280 x
+    // 1536 FP16 18.2 -> 14.1 us, 4096 x 512 x 4096 48.6 -> 37.9 us; below 1024 no gain: 4096 x 512 x 784 INT8 12.5 / 13.0 us)
+    const bool deep = (aligned || words) && g.kper == 0 && L.K >= 1024u;
     auto go = [&](auto tm_c, auto tn_c) {
         constexpr int TM = decltype(tm_c)::value, TN = decltype(tn_c)::value;
         const dim3 grid(tiles(64 * TM, 64 * TN), g.ksplits * halves);
+        if constexpr (TM == 1) {
+            if (deep) {
+                if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
+                    if (words) {
+                        sp_gemm16<FMT, F16T, TM, TN, true, true, 128><<<grid, 256, 0, g_stream>>>(g);
+                        return;
+                    }
+                }
+                sp_gemm16<FMT, F16T, TM, TN, true, false, 128><<<grid, 256, 0, g_stream>>>(g);
+                return;
+            }
+        }
         if constexpr (FMT == I8 || FMT == I4 || FMT == I2) {
             if (words) {
                 sp_gemm16<FMT, F16T, TM, TN, true, true><<<grid, 256, 0, g_stream>>>(g);

@@ -117,16 +117,18 @@ __device__ __forceinline__ void unpack_word16(uint32_t w, uint32_t *o)
     }
 }
 
-// Tile: BM x BN x 64, 256 threads = 2 x 2 waves, each wave TM x TN tiles of 32x32.
+// Tile: BM x BN x BK (BK = 64, or 128 for a K of 1024 and more), 256 threads = 2 x 2 waves, each wave TM x TN tiles of
+// 32x32.  A K split (g.kper, whole tiles of 64) goes with BK = 64 only.
 // LDS rows are padded by 8 elements so that 128-bit fragment reads of 32
 // consecutive rows spread over the banks.
 // W4 (integer codes, ALIGNED activations): the weight rows are whole 32-bit words but not whole 16-byte units
 // (784 INT4 codes = 392 bytes): the codes are fetched a word at a time instead of element by element.
-template <int FMT, bool F16T, int TM, int TN, bool ALIGNED, bool W4 = false>
+template <int FMT, bool F16T, int TM, int TN, bool ALIGNED, bool W4 = false, int BK = 64>
 __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
 {
     static_assert(!W4 || (ALIGNED && (FMT == I8 || FMT == I4 || FMT == I2)), "word loads: integer codes, aligned activations");
-    constexpr int BM = 64 * TM, BN = 64 * TN, BK = 64, LDK = BK + 8;
+    constexpr int BM = 64 * TM, BN = 64 * TN, LDK = BK + 8;
+    constexpr int KCH = BK / 8;                     // 16-byte pieces of a tile row of activations
     constexpr int bits = fmt_bits(FMT);
     constexpr int EPL = 128 / bits;                 // weight elements per 16-byte load
     constexpr int W_LOADS = (BN * BK / EPL + 255) / 256;
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
         if constexpr (ALIGNED) {
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
-                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                const int c = t + 256 * i, row = c / KCH, kc = c % KCH;
                 const uint32_t m = m0 + row < M ? m0 + row : M - 1;
                 const uint32_t k = k0 + kc * 8;
                 ra[i] = k < K ? *reinterpret_cast<const uint4 *>(A + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
@@ -209,7 +211,7 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
         if constexpr (ALIGNED) {
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
-                const int c = t + 256 * i, row = c >> 3, kc = c & 7;
+                const int c = t + 256 * i, row = c / KCH, kc = c % KCH;
                 *reinterpret_cast<uint4 *>(&As[row * LDK + kc * 8]) = ra[i];
             }
             if constexpr (W4) {

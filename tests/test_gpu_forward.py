@@ -608,7 +608,8 @@ def _decoded_layer(S, fmt, N, K, seed):
     # few outputs, activations streamed
     ("i8", 10, 1000, 256), ("i8", 10, 1000, 4096), ("i4", 64, 512, 1000), ("i2", 33, 2048, 513),
     ("bf16", 10, 1000, 300), ("f16", 7, 72, 65), ("i4", 10, 4096, 5),
-    # a few hundred samples: 256 x 256 tiles with K split over the grid
+    # a few hundred samples: 256 x 256 tiles with K split over the grid (K of 4096 and more), else the single-stage kernel
+    ("i8", 1024, 4096, 700), ("bf16", 2048, 4168, 300),
     ("bf16", 768, 1024, 130), ("f16", 512, 2048, 200), ("bf16", 1024, 1024, 255),
     ("bf16", 4096, 2048, 65), ("f16", 3000, 4096, 100), ("bf16", 4096, 8192, 128), ("i8", 8192, 2048, 129),
     ("i4", 1024, 2048, 300), ("bf16", 768, 1024, 513), ("i2", 2048, 4096, 1000), ("f16", 512, 1024, 257), ("i8", 1280, 1536, 600),
@@ -637,6 +638,11 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     # integer rows that are whole 32-bit words but not whole 16-byte units (784 INT4 codes = 392 bytes): word loads
     ("i4", 512, 784, 2048), ("i2", 300, 784, 2000), ("i8", 1000, 776, 600), ("i4", 520, 1000, 1100), ("i2", 2048, 1008, 2048),
     ("i4", 70, 24, 8), ("i8", 4096, 72, 4096),
+    # K of 1024 and more: K tiles of 128 (layers of up to 2 M weights and K below 4096 stay here instead of splitting K
+    # for the 256 x 256 tiles); K tails of 120, 64 and 16 elements, word loads
+    ("f16", 1024, 1024, 2048), ("i8", 512, 2048, 4096), ("i4", 520, 1040, 1100), ("bf16", 768, 2040, 3000), ("i2", 1000, 1088, 1800),
+    ("f16", 2000, 1000, 2100), ("i4", 2080, 1056, 300), ("i8", 1100, 2000, 700), ("f16", 2001, 1032, 2100),
+    ("bf16", 8192, 1000, 100), ("f16", 5000, 1160, 77),
 ])
 def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
@@ -678,11 +684,11 @@ def test_small_layers_run_in_one_launch(S, fmt, N, K, n):
     # Enough tiles for the chip (tails of 40, 8, 48 and 32 elements) ...
     ("bf16", 4096, 1000, 4096), ("f16", 4096, 1096, 3000), ("i8", 4096, 1008, 4096), ("i4", 4096, 1056, 4096),
     # ... K split over the grid, the partial tile in the last split ...
-    ("f16", 2000, 1000, 2100), ("bf16", 2048, 1000, 4096), ("i4", 2080, 1056, 300), ("i8", 1100, 2000, 700),
-    # ... a single row of 128 x 256 tiles, ragged in M and N, and a K of two tiles and a bit
-    ("bf16", 8192, 1000, 100), ("f16", 5000, 1160, 77), ("bf16", 8200, 136, 8200),
+    ("f16", 2200, 4200, 2100), ("bf16", 2048, 1000, 4096), ("i4", 2080, 4128, 300), ("i8", 1100, 4112, 700),
+    # ... a single row of 128 x 256 tiles (K split from K = 3072), ragged in M and N, and a K of two tiles and a bit
+    ("bf16", 8192, 3080, 100), ("f16", 5000, 4136, 77), ("bf16", 8200, 136, 8200),
     # output rows that are not whole 16-byte units: one element per lane and store, with and without a K split
-    ("bf16", 4099, 1024, 4096), ("f16", 2001, 1032, 2100), ("i8", 4102, 1040, 3000),
+    ("bf16", 4099, 1024, 4096), ("f16", 2101, 4104, 2100), ("i8", 4102, 1040, 3000),
 ])
 def test_big_tile_gemm_takes_a_partial_k_tile(S, fmt, N, K, n):
     net, W, b = _decoded_layer(S, fmt, N, K, seed=N + 3 * K + n)
@@ -847,7 +853,8 @@ def _same_nonfinite(got, want):
     ("i4", 16384, 2048, 8, 0, "sp_skinny16_kw"), ("i8", 2100, 2064, 48, 0, "sp_skinny16"),
     ("f16", 1500, 4096, 60, 0, "sp_skinny16"), ("bf16", 10, 1000, 300, 0, "sp_skinny16_kw"),
     ("f16", 1500, 1000, 77, 0, "sp_gemm16_small"), ("i2", 600, 1000, 200, 0, "sp_gemm16_small"),
-    ("bf16", 2048, 2048, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
+    ("bf16", 2048, 4096, 600, 0, "sp_gemm16_big"), ("i2", 2048, 4096, 1000, 0, "sp_gemm16_big"),
+    ("bf16", 2048, 2048, 600, 0, "sp_gemm16"),
     ("i8", 1000, 528, 700, 0, "sp_gemm16"), ("i4", 257, 100, 513, 0, "sp_gemm16"),
 ])
 def test_infinities_and_nans_travel_like_in_fp32(S, fmt, N, K, n, flags, kernel):
