@@ -1220,17 +1220,17 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
     }
 }
 
-// Layers that run in one launch of sp_gemm16_small: more than 8 samples (fewer take one launch of sp_skinny16_kw), more
-// than 64 outputs (fewer stream the activations), at most 512 tiles of 32 x 32, K up to 2048 (its eight waves are all
-// the K split there is), and tiles x K up to 512 K: every tile reads 64 rows of K elements from L2.  Measured, whole
-// nets, against the streaming / tiled kernels with their K split over the grid, second launch and separate conversion
-// of the input: 784-512-1000-10 INT8 at 16 / 256 / 512 samples 16.5 / 18.9 / 22.3 against 24.8 / 29.8 / 28.0 us, eight
-// 256 x 256 layers at 64 / 1024 samples 31 / 35 against 51 / 49 us, three 1024 x 1024 layers at 256 samples 24 against
-// 38 us, at 512 samples (512 tiles x 1024) 40 against 41 us; beyond the bound it loses: two 2048 x 2048 layers at 256
-// samples (512 tiles x 2048) 46 against 35 us.
+// Layers that run in one launch of sp_gemm16_small: more than 64 outputs (fewer stream the activations), at most 512
+// tiles of 32 x 32, K up to 2048 (its eight waves are all the K split there is), and tiles x K up to 512 K: every tile
+// reads 64 rows of K elements from L2.  Measured, whole nets, against the streaming / tiled kernels with their K split
+// over the grid, second launch and separate conversion of the input: 784-512-1000-10 INT8 at 16 / 256 / 512 samples
+// 16.5 / 18.9 / 22.3 against 24.8 / 29.8 / 28.0 us, FP16 at 5 samples 16 against 23 us; eight 256 x 256 layers at 5 / 64 /
+// 1024 samples 25 / 31 / 35 against 42 / 51 / 49 us, three 1024 x 1024 layers at 256 samples 24 against 38 us, at 512
+// samples (512 tiles x 1024) 40 against 41 us; beyond the bound it loses: two 2048 x 2048 layers at 256 samples (512
+// tiles x 2048) 46 against 35 us.
 bool gemm16_small_layer(uint32_t M, uint32_t N, uint32_t K, uint32_t halves)
 {
-    if (halves != 1u || K % 8u != 0 || K > 2048u || N <= 64u || M <= 8u) return false;
+    if (halves != 1u || K % 8u != 0 || K > 2048u || N <= 64u) return false;
     const uint64_t tiles = (uint64_t)((M + 31u) / 32u) * ((N + 31u) / 32u);
     return tiles <= 512u && tiles * K <= (512u << 10);
 }

@@ -637,7 +637,7 @@ def test_thin_and_split_k_shapes(S, fmt, N, K, n):
     ("i8", 300, 1000, 1800), ("i4", 257, 100, 513), ("i2", 1030, 1000, 520), ("i8", 200, 1000, 2400),
     # integer rows that are whole 32-bit words but not whole 16-byte units (784 INT4 codes = 392 bytes): word loads
     ("i4", 512, 784, 2048), ("i2", 300, 784, 2000), ("i8", 1000, 776, 600), ("i4", 520, 1000, 1100), ("i2", 2048, 1008, 2048),
-    ("i4", 70, 24, 8), ("i8", 4096, 72, 4096),
+    ("i4", 70, 24, 6000), ("i8", 4096, 72, 4096),
     # K of 1024 and more: K tiles of 128 (layers of up to 2 M weights and K below 4096 stay here instead of splitting K
     # for the 256 x 256 tiles); K tails of 120, 64 and 16 elements, word loads
     ("f16", 1024, 1024, 2048), ("i8", 512, 2048, 4096), ("i4", 520, 1040, 1100), ("bf16", 768, 2040, 3000), ("i2", 1000, 1088, 1800),
@@ -657,11 +657,12 @@ def test_single_stage_gemm_tile_shapes(S, fmt, N, K, n):
 
 @pytest.mark.parametrize("fmt,N,K,n", [
     # up to 512 tiles of 32 x 32 and K up to 2048: ragged edges in both directions, K tails of 8, 16 and 24 elements
-    # (K = 1000, 784, 24, 72), a K shorter than the eight waves' shares, every weight format, 9 samples and up
+    # (K = 1000, 784, 24, 72), a K shorter than the eight waves' shares, every weight format, 5 samples and up
     ("bf16", 512, 784, 600), ("i8", 300, 1000, 700), ("i8", 200, 1000, 512), ("i4", 512, 784, 1024), ("i2", 300, 784, 300),
     ("i4", 520, 1000, 64), ("i4", 70, 24, 9), ("f16", 1500, 1000, 77), ("i2", 1000, 320, 130), ("bf16", 4096, 2048, 40),
     ("i8", 512, 784, 256), ("i8", 1000, 512, 256), ("f16", 65, 8, 9), ("i2", 97, 2048, 33), ("bf16", 16384, 32, 32),
     ("i8", 256, 256, 2048), ("f16", 1024, 1024, 512), ("i4", 2048, 2048, 128), ("i2", 130, 72, 1000),
+    ("i8", 1000, 512, 5), ("f16", 512, 784, 8), ("i2", 8192, 256, 6), ("bf16", 100, 2048, 7),
 ])
 def test_small_layers_run_in_one_launch(S, fmt, N, K, n):
     """Layers of a few hundred 32 x 32 output tiles run in one launch whose workgroups split K among their waves and
