@@ -34,7 +34,7 @@ def _net(S, fmt, topo, acts, seed):
 
 CASES = [
     # fmt, topology, activations, (first n, second smaller n), flags
-    ("i8", [784, 512, 1000, 10], ["relu", "relu", "softmax"], (4096, 300), 0),     # tiled GEMMs, classifier head
+    ("i8", [784, 512, 1000, 10], ["relu", "relu", "softmax"], (4096, 300), 0),     # tiled GEMMs, classifier head; at 300 the one-launch small-layer kernel
     ("i8", [784, 512, 1000, 10], ["relu", "relu", "softmax"], (4, 1), 0),          # vector kernels
     ("i4", [1024, 4096, 4096, 512], ["relu", "tanh", "none"], (64, 8), 0),         # streaming kernels, K splits + reduce
     ("i4", [1024, 4096, 4096, 512], ["relu", "tanh", "none"], (3, 2), 0),          # self-quantising integer GEMV
