@@ -1398,6 +1398,25 @@ uint32_t gemm32_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
     return (ktiles + per - 1) / per;
 }
 
+// The forward products' K splits.  From 512 tiles on, and from 256 tiles on when K is below 1024 (a short kernel, on
+// which the second launch and the partial sums weigh most), the split costs more than idle compute units do: forward
+// of one layer, no split against the rule above, 4096 x 512 x 784 40 against 48 us, 2048 x 1000 x 512 29 against 37 us,
+// 1024 x 1000 x 512 19 against 26 us, 4096 x 256 x 256 11 against 21 us, 3000 x 1000 x 2000 135 against 142 us, four 512 x 512
+// layers at 2048 / 4096 samples 67 / 106 against 105 / 149 us; but 256 to 511 tiles with a longer K keep it (130 x 8192 x
+// 1024 46 against 56 us, 200 x 4096 x 1100 36 against 48 us, 700 x 2048 x 1536 63 against 72 us, 1500 x 1024 x 1024 47 against
+// 50 us), and so do rows that are not whole 16-byte units, whose element-wise loads make every tile slow and an uneven
+// last round expensive (4096 x 257 x 999).  Fewer than 256 tiles: as above (300 x 2048 x 2048 68 us unsplit, 42 us split
+// seven ways).
+uint32_t gemm32_fwd_splits(uint32_t M, uint32_t N, uint32_t K, uint32_t *kper)
+{
+    const uint32_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    if (K % 4u == 0 && (tiles >= 512u || (tiles >= 256u && K < 1024u))) {
+        *kper = (K + 31u) / 32u * 32u;
+        return 1;
+    }
+    return gemm32_splits(M, N, K, kper);
+}
+
 // FP32 layers of at most 64 outputs are one row of tiles at most; with up to eight samples, one pass of the vector
 // kernel (a workgroup per row), that kernel is quicker than the matrix-core kernel and its reduction launch
 // (16384 -> 64 -> 10 at 5 / 8 samples: 24 / 25 against 43 us; 8192 -> 10: 13 against 23 us; at 16 samples, two passes,
@@ -1428,7 +1447,7 @@ bool launch_gemm32(const LayerArgs &L, const float *A, float *C, uint32_t M, flo
         sp_gemm32_f32_big<<<((M + 127u) / 128u) * ((L.N + 127u) / 128u), 256, lds, g_stream>>>(g);
         return false;
     }
-    uint32_t splits = gemm32_splits(M, L.N, L.K, &g.kper);
+    uint32_t splits = gemm32_fwd_splits(M, L.N, L.K, &g.kper);
     // small layers that would need a K split and a second launch: one launch of 32 x 32 tiles, K split inside the
     // workgroup (measured against the split path: 256 x 512 x 784 8 against 12 us, 1024 x 512 x 784 17 against 20 us;
     // beyond 512 tiles or K = 1024 the split path is the faster one: 1024 x 1024 x 1024 42 against 32 us)
@@ -1512,7 +1531,7 @@ WorkspaceNeed workspace_need(const sphip_net *net, uint32_t n, uint32_t flags)
             }
         } else if (net->prec == F32) {
             if (reg == R_GEMV) continue;
-            const uint32_t sp = gemm32_splits(n, N, K, &kper);
+            const uint32_t sp = gemm32_fwd_splits(n, N, K, &kper);
             if (sp > 1) ws = (uint64_t)sp * n * N;
         } else {
             const ThinPlan tp = plan_thin(net->prec, n, N, K);
