@@ -331,8 +331,41 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
     // epilogue: scale, bias, activation, store.  Sigmoid and tanh have a copy of the loops to themselves: a switch
     // over all activations behind every one of a lane's outputs is mostly their code, fetched for nothing.
     const float wscale = g.L.wscale;
+    // 16-bit outputs in rows of whole 16-byte units: a wave turns each 32 x 32 block around in LDS (the tiles' memory,
+    // free once every wave has read its last fragments) and stores 16 bytes per lane, two store instructions per
+    // block instead of sixteen two-byte ones
+    const bool rows16 = !g.out_f32 && N % 8u == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15u) == 0;     // (uniform)
+    if (rows16) __syncthreads();
+    constexpr int SP = 40;                                   // row pitch of a wave's 32 x 32 staging block, elements
+    uint16_t *const stage = (wave < 2 ? As : Ws) + (wave & 1) * (32 * SP);
     auto emit = [&](auto slow_c) __attribute__((always_inline)) {
         constexpr bool SLOW = decltype(slow_c)::value;
+        if (rows16) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+                const float bias = elem_value_rt(g.L.bias_fmt, g.L.bias, col < N ? col : N - 1) * g.L.bscale;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float pre = fmaf(acc[i][j][r], wscale, bias);
+                        const float v = SLOW ? apply_act(pre, g.L.act) : apply_act_cheap(pre, g.L.act);
+                        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * SP + (lane & 31)] = f32_to_t16<F16T>(v);
+                    }
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int p = 0; p < 2; ++p) {
+                        const int rr = (lane >> 2) + 16 * p, ch = lane & 3;
+                        const uint4 d = *reinterpret_cast<const uint4 *>(&stage[rr * SP + ch * 8]);
+                        const uint32_t row = m0 + wm * TM * 32 + i * 32 + rr, c0 = n0 + wn * TN * 32 + j * 32 + ch * 8;
+                        if (row < M && c0 < N) *reinterpret_cast<uint4 *>(reinterpret_cast<uint16_t *>(g.C) + (size_t)row * N + c0) = d;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const uint32_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
