@@ -1230,9 +1230,10 @@ void launch_thin(SkinnyArgs a, const ThinPlan &p)
 // tiles x 2048) 46 against 35 us.
 bool gemm16_small_layer(uint32_t M, uint32_t N, uint32_t K, uint32_t halves)
 {
-    if (halves != 1u || K % 8u != 0 || K > 2048u || N <= 64u) return false;
+    if (K % 8u != 0 || K > 2048u || N <= 64u) return false;
     const uint64_t tiles = (uint64_t)((M + 31u) / 32u) * ((N + 31u) / 32u);
-    return tiles <= 512u && tiles * K <= (512u << 10);
+    // (split activations: two activation matrices against one of weights, a tile reads 96 rows instead of 64)
+    return tiles <= 512u && tiles * K * (1u + halves) <= (1024u << 10);
 }
 
 template <int FMT, bool F16T>
@@ -1244,6 +1245,13 @@ void launch_gemm16_fmt(const LayerArgs &L, const uint16_t *A, void *C, uint32_t 
         tl_route.name = "sp_gemm16_small";
         if (tl_route.dry) return;
         const uint32_t grid = ((M + 31u) / 32u) * ((L.N + 31u) / 32u);
+        if constexpr (F16T) {
+            if (halves == 2) {
+                if (ctx.x_f32) sp_gemm16_small<FMT, F16T, true, 2><<<grid, 512, 0, g_stream>>>(g);
+                else sp_gemm16_small<FMT, F16T, false, 2><<<grid, 512, 0, g_stream>>>(g);
+                return;
+            }
+        }
         if (ctx.x_f32) sp_gemm16_small<FMT, F16T, true><<<grid, 512, 0, g_stream>>>(g);
         else sp_gemm16_small<FMT, F16T, false><<<grid, 512, 0, g_stream>>>(g);
         return;
@@ -1677,12 +1685,12 @@ int enqueue_forward(sphip_net *net, const Workspace &wk, const float *d_x, uint3
     const void *in = d_x;
     const bool x_fused = reg == R_GEMM16 && gemm16_small_layer(n, net->topo[1], net->topo[0], tl_route.halves) &&
                          (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0;
-    if (split && !only_layer) {
+    if (x_fused) {
+        // (the first layer's kernel rounds, or splits, the FP32 input itself)
+    } else if (split && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         sp_cvt16_split<<<(uint32_t)((cnt / 4 + 255) / 256 + 1), 256, 0, g_stream>>>(d_x, (uint16_t *)wk.buf[1], cnt);
         in = wk.buf[1];
-    } else if (x_fused) {
-        // (the first layer's kernel rounds the FP32 input itself)
     } else if (reg == R_GEMM16 && !only_layer) {
         const uint64_t cnt = (uint64_t)n * net->topo[0];
         const uint32_t grid = (uint32_t)((cnt / 4 + 255) / 256 + 1);

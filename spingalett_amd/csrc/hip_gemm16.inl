@@ -395,11 +395,14 @@ __global__ __launch_bounds__(256) void sp_gemm16(const GemmArgs g)
 // k = 32 s + 16 h .. + 15 of row r of both operands straight into registers, as two pieces of eight (K % 8 == 0: a piece
 // is inside its row or beyond it), and feeds a piece of each operand to one MFMA (a sum over k in any order).  For
 // outputs of a few hundred tiles, where the streaming and the tiled kernels need a K split over the grid and a second
-// launch to fill the chip.  XF32: the activations are still the caller's FP32 input, rounded here as sp_cvt16 would
-// (g.A then points at floats).
-template <int FMT, bool F16T, bool XF32>
+// launch to fill the chip.  XF32: the activations are still the caller's FP32 input, rounded here as sp_cvt16 (or, with
+// split activations, sp_cvt16_split) would (g.A then points at floats).  HALVES == 2: split activations, two FP16
+// matrices hi and lo = (a - hi) 2^11, M K elements apart; a second accumulator takes the lo products, a wave adds it,
+// times 2^-11, to its hi sum, and 16-bit outputs leave as the two matrices of the next layer's input.
+template <int FMT, bool F16T, bool XF32, int HALVES = 1>
 __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
 {
+    static_assert(HALVES == 1 || F16T, "split activations are FP16");
     constexpr int NW = 8, U = 2;
     constexpr int bits = fmt_bits(FMT);
     constexpr int PB = bits;                           // bytes of a piece of eight weights
@@ -415,7 +418,7 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
     const float *ap32 = reinterpret_cast<const float *>(g.A) + (size_t)am * K + 16 * h;
     const uint8_t *wp = g.L.w + (size_t)wn * ((size_t)K * bits / 8u) + (size_t)(2 * h) * PB;
 
-    struct Frag { uint4 a[2], w[2]; };
+    struct Frag { uint4 a[2], al[HALVES == 2 ? 2 : 1], w[2]; };
     auto ld = [&](uint32_t s) -> Frag {
         Frag f;
 #pragma unroll
@@ -424,12 +427,25 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
             if constexpr (XF32) {
                 const float4 lo = ok ? *reinterpret_cast<const float4 *>(ap32 + 32u * s + 8 * p) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 const float4 hi = ok ? *reinterpret_cast<const float4 *>(ap32 + 32u * s + 8 * p + 4) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                f.a[p].x = (uint32_t)f32_to_t16<F16T>(lo.x) | ((uint32_t)f32_to_t16<F16T>(lo.y) << 16);
-                f.a[p].y = (uint32_t)f32_to_t16<F16T>(lo.z) | ((uint32_t)f32_to_t16<F16T>(lo.w) << 16);
-                f.a[p].z = (uint32_t)f32_to_t16<F16T>(hi.x) | ((uint32_t)f32_to_t16<F16T>(hi.y) << 16);
-                f.a[p].w = (uint32_t)f32_to_t16<F16T>(hi.z) | ((uint32_t)f32_to_t16<F16T>(hi.w) << 16);
+                if constexpr (HALVES == 2) {
+                    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                    uint16_t eh[8], el[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) split_f16(v[e], eh[e], el[e]);
+                    f.a[p] = make_uint4((uint32_t)eh[0] | ((uint32_t)eh[1] << 16), (uint32_t)eh[2] | ((uint32_t)eh[3] << 16),
+                                        (uint32_t)eh[4] | ((uint32_t)eh[5] << 16), (uint32_t)eh[6] | ((uint32_t)eh[7] << 16));
+                    f.al[p] = make_uint4((uint32_t)el[0] | ((uint32_t)el[1] << 16), (uint32_t)el[2] | ((uint32_t)el[3] << 16),
+                                         (uint32_t)el[4] | ((uint32_t)el[5] << 16), (uint32_t)el[6] | ((uint32_t)el[7] << 16));
+                } else {
+                    f.a[p].x = (uint32_t)f32_to_t16<F16T>(lo.x) | ((uint32_t)f32_to_t16<F16T>(lo.y) << 16);
+                    f.a[p].y = (uint32_t)f32_to_t16<F16T>(lo.z) | ((uint32_t)f32_to_t16<F16T>(lo.w) << 16);
+                    f.a[p].z = (uint32_t)f32_to_t16<F16T>(hi.x) | ((uint32_t)f32_to_t16<F16T>(hi.y) << 16);
+                    f.a[p].w = (uint32_t)f32_to_t16<F16T>(hi.z) | ((uint32_t)f32_to_t16<F16T>(hi.w) << 16);
+                }
             } else {
                 f.a[p] = ok ? *reinterpret_cast<const uint4 *>(ap16 + 32u * s + 8 * p) : make_uint4(0, 0, 0, 0);
+                if constexpr (HALVES == 2)
+                    f.al[p] = ok ? *reinterpret_cast<const uint4 *>(ap16 + (size_t)M * K + 32u * s + 8 * p) : make_uint4(0, 0, 0, 0);
             }
             const uint8_t *src = wp + (size_t)s * (4 * PB) + p * PB;
             if constexpr (FMT == F16 || FMT == BF16) {
@@ -445,9 +461,9 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
         }
         return f;
     };
-    f32x16 acc;
+    f32x16 acc, accl;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = accl[r] = 0.0f;
     auto fma2 = [&](const Frag &f) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -471,6 +487,10 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
                 __builtin_memcpy(&a, &f.a[p], 16);
                 __builtin_memcpy(&b, &wv, 16);
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+                if constexpr (HALVES == 2) {
+                    __builtin_memcpy(&a, &f.al[p], 16);
+                    accl = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, accl, 0, 0, 0);
+                }
             } else {
                 bf16x8 a, b;
                 __builtin_memcpy(&a, &f.a[p], 16);
@@ -489,7 +509,8 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
     }
     for (; s < s1; ++s) fma2(ld(s));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) part[wave][(8 * (r >> 2) + 4 * h + (r & 3)) * 33 + q] = acc[r];
+    for (int r = 0; r < 16; ++r)
+        part[wave][(8 * (r >> 2) + 4 * h + (r & 3)) * 33 + q] = HALVES == 2 ? fmaf(accl[r], kLoScale, acc[r]) : acc[r];
     __syncthreads();
     // the waves' sums in wave order, scale, bias, activation; 512 threads, two outputs each
     const float wscale = g.L.wscale;
@@ -503,7 +524,12 @@ __global__ __launch_bounds__(512) void sp_gemm16_small(const GemmArgs g)
         v = apply_act(fmaf(v, wscale, elem_value_rt(g.L.bias_fmt, g.L.bias, n0 + col) * g.L.bscale), g.L.act);
         const size_t o = (size_t)(m0 + row) * N + n0 + col;
         if (g.out_f32) reinterpret_cast<float *>(g.C)[o] = v;
-        else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
+        else if constexpr (HALVES == 2) {
+            uint16_t eh, el;
+            split_f16(v, eh, el);
+            reinterpret_cast<uint16_t *>(g.C)[o] = eh;
+            reinterpret_cast<uint16_t *>(g.C)[(size_t)M * N + o] = el;
+        } else reinterpret_cast<uint16_t *>(g.C)[o] = f32_to_t16<F16T>(v);
     }
 }
 

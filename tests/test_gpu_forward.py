@@ -406,6 +406,8 @@ def test_split_activations_reach_the_argmax_bar_on_every_head(S, O, fmt, topo, a
     ([256, 384, 520, 33], ["sigmoid", "softmax", "none"], 300),   # hidden softmax, streaming kernels, odd widths
     ([77, 130, 65], ["leaky_relu", "foo52"], 129),                # rows that are not whole 16-byte units
     ([512, 1024, 512, 1000], ["relu", "leaky_relu", "softmax"], 2048),   # tiled GEMM with and without K splits
+    ([784, 512, 1000, 10], ["relu", "relu", "softmax"], 256),            # small layers in one launch, FP32 input split in it
+    ([1000, 136, 2048, 72], ["tanh", "sigmoid", "none"], 70),            # the same with K tails and ragged tiles
 ])
 def test_split_activations_on_every_kernel_family(S, O, fmt, topo, acts, n):
     """The split-activation forward through every matrix-core kernel family (streaming with the weights or the
