@@ -39,12 +39,18 @@ def readings(directory: str, counter: str):
 
 
 def dominant(rows, kernel: str):
-    vals = [v for k, v in rows if kernel in k]
-    if not vals:
+    """Mean reading and count of the dominant layer's launches: among the dispatches of `kernel`, the group (same
+    instantiation, readings within a few percent) that was launched most often.  bench.py times the dominant layer with
+    many extra launches of its own, so it outnumbers every other layer that runs a kernel of the same name."""
+    import math
+    groups = {}
+    for k, v in rows:
+        if kernel in k:
+            groups.setdefault((k, round(math.log(max(v, 1e-9)) * 16)), []).append(v)
+    if not groups:
         raise SystemExit(f"no dispatch of {kernel} in the counter files")
-    top = max(vals)
-    near = [v for v in vals if v >= 0.8 * top]
-    return sum(near) / len(near), len(near)
+    vals = max(groups.values(), key=lambda g: (len(g), sum(g)))
+    return sum(vals) / len(vals), len(vals)
 
 
 def copy_reading(rows):
@@ -64,6 +70,7 @@ def main():
     ap.add_argument("--launches", type=int, default=1,
                     help="launches of the kernel per forward of the layer (a batch that runs in blocks of rows: bench.py "
                          "reports it as roofline_kernel.launches); the entry holds their sum")
+    ap.add_argument("--no-alt", action="store_true", help="the counter runs were made with bench.py --no-alt (recorded in the entry's commands)")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles", "traffic.json"))
     args = ap.parse_args()
 
@@ -90,10 +97,11 @@ def main():
         "bytes": int(round((fetch * f_factor + write * w_factor) * 1024)) * args.launches,
         "commands": [
             f"rocprofv3 --pmc {c} -d out/{d} -o p --output-format csv -- python3 bench.py --workload {args.workload} "
-            f"--batch {args.batch} --steps 40 --warmup 5 --no-extra --no-cpu --calibrate-copy"
+            f"--batch {args.batch} --steps 40 --warmup 5 --no-extra --no-cpu{' --no-alt' if args.no_alt else ''} --calibrate-copy"
             for c, d in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write"))
         ] + [f"python3 bench_traffic.py --workload {args.workload} --batch {args.batch} --kernel {args.kernel} "
-             "--fetch out/fetch --write out/write" + (f" --launches {args.launches}" if args.launches > 1 else "")],
+             "--fetch out/fetch --write out/write" + (f" --launches {args.launches}" if args.launches > 1 else "") +
+             (" --no-alt" if args.no_alt else "")],
     }
     try:
         with open(args.out) as f:
